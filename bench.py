@@ -1,0 +1,250 @@
+"""Benchmark of the fused layer ops on the Llama-3-8B 2304-token hybrid batch (one MI355X).
+
+A "step" is one pass of a decoder layer's element-wise chain over one hybrid batch
+(2048 prefill tokens + 256 decode tokens), in layer order:
+
+    fused_add_rms_norm [2304, 4096]            (input layernorm with the residual add fused in)
+    rotary_embedding   q [2304, 32*128], k [2304, 8*128], views of a packed [2304, 6144] qkv
+    fused_add_rms_norm [2304, 4096]            (post-attention layernorm)
+    silu_and_mul       [2304, 2*14336] -> [2304, 14336]
+
+All inputs are resident in HBM before the timed region.  Every step works on a different one of
+several independent buffer sets whose total footprint exceeds 512 MB, so the 256 MB Infinity Cache
+cannot serve the reads ("cold" numbers).  `value` is the step's algorithmic bytes divided by the
+step time.  `per_op` carries, for every op (plus rms_norm alone and the Mixtral-shaped MoE routing
+ops), µs per call, GB/s and fraction of the 8 TB/s HBM peak, cold and warm (same buffers every
+call).  `roofline` describes the dominant kernel of the step, silu_and_mul, timed with HIP events
+placed around that launch inside the timed region.  `cpu_baseline` is the PyTorch CPU formulation
+of the same step on this machine's host cores.
+
+Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "sarathi-serve_amd"), os.path.join(ROOT, "tests")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0
+
+T, H, NQ, NKV, D, DFF = 2304, 4096, 32, 8, 128, 14336
+PREFILL = 2048
+BF16 = 2
+
+# algorithmic (compulsory) bytes per call: every input element read once, every output element
+# written once, in-place tensors counted read + write, weight / touched cache rows once
+BYTES = {
+    "fused_add_rms_norm": 4 * T * H * BF16 + H * BF16,
+    "rms_norm": 2 * T * H * BF16 + H * BF16,
+    "rotary_embedding": 2 * (T * NQ * D + T * NKV * D) * BF16 + T * 8,   # + touched cache rows
+    "silu_and_mul": (2 * T * DFF + T * DFF) * BF16,
+}
+MOE_T, MOE_E, MOE_K, MOE_B = 4096, 8, 2, 64
+BYTES["topk_softmax"] = MOE_T * MOE_E * 4 + 3 * MOE_T * MOE_K * 4
+_moe_sorted = MOE_T * MOE_K + MOE_E * (MOE_B - 1)
+BYTES["moe_align_block_size"] = MOE_T * MOE_K * 4 + _moe_sorted * 4 + 4 * (
+    (_moe_sorted + MOE_B - 1) // MOE_B) + 4
+
+
+def make_set(torch, g, dev, cache_cpu):
+    """One independent set of step inputs (seeded on the CPU, fp32 draw -> bf16)."""
+    from helpers import hybrid_positions, randn
+    s = {}
+    s["x"] = randn((T, H), g).to(dev)
+    s["res"] = randn((T, H), g).to(dev)
+    s["w1"] = randn((H,), g, mean=1.0, std=0.1).to(dev)
+    s["w2"] = randn((H,), g, mean=1.0, std=0.1).to(dev)
+    s["qkv"] = randn((T, (NQ + 2 * NKV) * D), g).to(dev)
+    s["q"], s["k"], _ = s["qkv"].split([NQ * D, NKV * D, NKV * D], dim=-1)
+    s["pos"] = hybrid_positions(T, PREFILL, g).to(dev)
+    s["cache"] = cache_cpu.to(dev)
+    s["gate_up"] = randn((T, 2 * DFF), g).to(dev)
+    s["act"] = torch.empty((T, DFF), dtype=torch.bfloat16, device=dev)
+    s["norm_out"] = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    return s
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--sets", type=int, default=4, help="independent buffer sets to rotate through")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this op library runs on one GPU; --gpus must be 1 "
+                 "(the ops are per-token and never communicate)")
+
+    import torch
+    import sarathi_amd as ops          # raises if the HIP extension is missing
+    from helpers import THETA_LLAMA3, cos_sin_cache, gen
+    from oracle import torch_formulations as cpu_ops
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    LN, ACT, ROPE, MOE = ops.layernorm_ops, ops.activation_ops, ops.pos_encoding_ops, ops.moe_ops
+
+    g = gen(1)
+    cache_cpu = cos_sin_cache(8192, D, THETA_LLAMA3, torch.bfloat16)
+    sets = [make_set(torch, g, dev, cache_cpu) for _ in range(args.sets)]
+    set_bytes = sum(v.numel() * v.element_size() for k, v in sets[0].items() if k not in ("q", "k"))
+
+    def step(s, ev=None):
+        LN.fused_add_rms_norm(s["x"], s["res"], s["w1"], 1e-5)
+        ROPE.rotary_embedding(s["pos"], s["q"], s["k"], D, s["cache"], True)
+        LN.fused_add_rms_norm(s["x"], s["res"], s["w2"], 1e-5)
+        if ev is not None:
+            ev[0].record()
+        ACT.silu_and_mul(s["act"], s["gate_up"])
+        if ev is not None:
+            ev[1].record()
+
+    step_bytes = 2 * BYTES["fused_add_rms_norm"] + BYTES["rotary_embedding"] + BYTES["silu_and_mul"]
+
+    # ---- the timed region: exactly --steps steps, rotating buffer sets (cold) ----
+    for i in range(args.warmup):
+        step(sets[i % len(sets)])
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+           for _ in range(args.steps)]
+    t0 = torch.cuda.Event(enable_timing=True)
+    t1 = torch.cuda.Event(enable_timing=True)
+    wall0 = time.perf_counter()
+    t0.record()
+    for i in range(args.steps):
+        step(sets[i % len(sets)], evs[i])
+    t1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - wall0
+    gpu_ms = t0.elapsed_time(t1)
+    ms_per_step = max(gpu_ms, wall * 1e3) / args.steps
+    silu_us = sum(a.elapsed_time(b) for a, b in evs) * 1e3 / args.steps
+
+    # ---- per-op tables: K back-to-back launches between two events ----
+    def time_op(fn, cold, reps):
+        n = len(sets) if cold else 1
+        for i in range(5):
+            fn(sets[i % n])
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for i in range(reps):
+            fn(sets[i % n])
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e3 / reps
+
+    mg = gen(3)
+    gating = torch.randn((MOE_T, MOE_E), generator=mg, dtype=torch.float32).to(dev)
+    tw = torch.empty((MOE_T, MOE_K), dtype=torch.float32, device=dev)
+    ti = torch.empty((MOE_T, MOE_K), dtype=torch.int32, device=dev)
+    ts = torch.empty((MOE_T, MOE_K), dtype=torch.int32, device=dev)
+    MOE.topk_softmax(tw, ti, ts, gating)
+    sorted_ids = torch.empty((_moe_sorted,), dtype=torch.int32, device=dev)
+    expert_ids = torch.empty(((_moe_sorted + MOE_B - 1) // MOE_B,), dtype=torch.int32, device=dev)
+    post_pad = torch.empty((1,), dtype=torch.int32, device=dev)
+
+    op_fns = {
+        "fused_add_rms_norm": lambda s: LN.fused_add_rms_norm(s["x"], s["res"], s["w1"], 1e-5),
+        "rms_norm": lambda s: LN.rms_norm(s["norm_out"], s["x"], s["w1"], 1e-5),
+        "rotary_embedding": lambda s: ROPE.rotary_embedding(s["pos"], s["q"], s["k"], D, s["cache"], True),
+        "silu_and_mul": lambda s: ACT.silu_and_mul(s["act"], s["gate_up"]),
+        "topk_softmax": lambda s: MOE.topk_softmax(tw, ti, ts, gating),
+        "moe_align_block_size": lambda s: MOE.moe_align_block_size_filled(
+            ti, MOE_E, MOE_B, sorted_ids, expert_ids, post_pad),
+    }
+    per_op = {}
+    for name, fn in op_fns.items():
+        row = {"bytes": BYTES[name]}
+        for label, cold in (("cold", True), ("warm", False)):
+            if name in ("topk_softmax", "moe_align_block_size") and cold:
+                continue   # 0.07-0.2 MB working sets: launch-latency-bound, one (warm) figure
+            us = time_op(fn, cold, max(args.steps, 50))
+            gbs = BYTES[name] / us * 1e-3
+            row[label] = {"us": round(us, 3), "GBps": round(gbs, 1),
+                          "frac_of_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        per_op[name] = row
+
+    silu_gbs = BYTES["silu_and_mul"] / silu_us * 1e-3
+    roofline = {
+        "kernel": "silu_and_mul_kernel (bf16, [2304, 28672] -> [2304, 14336])",
+        "bound": "hbm", "achieved": round(silu_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(silu_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+        "bytes_per_launch": BYTES["silu_and_mul"], "avg_launch_us": round(silu_us, 3),
+        "timing": "hipEvent pair around each launch inside the timed region, cold buffers",
+    }
+
+    # ---- CPU baseline: the PyTorch formulation of the same step on the host cores ----
+    cpu = None
+    if not args.no_cpu_baseline:
+        from helpers import hybrid_positions, randn
+        cg = gen(1)
+        cx, cr = randn((T, H), cg), randn((T, H), cg)
+        cw = randn((H,), cg, mean=1.0, std=0.1)
+        cqkv = randn((T, (NQ + 2 * NKV) * D), cg)
+        cq, ck, _ = cqkv.split([NQ * D, NKV * D, NKV * D], dim=-1)
+        cpos = hybrid_positions(T, PREFILL, cg)
+        cgu = randn((T, 2 * DFF), cg)
+        cact = torch.empty((T, DFF), dtype=torch.bfloat16)
+
+        def cpu_step():
+            cpu_ops.fused_add_rms_norm(cx, cr, cw, 1e-5)
+            cpu_ops.rotary_embedding(cpos, cq, ck, D, cache_cpu, True)
+            cpu_ops.fused_add_rms_norm(cx, cr, cw, 1e-5)
+            cpu_ops.silu_and_mul(cact, cgu)
+
+        cpu_step()
+        t_start = time.perf_counter()
+        cpu_step()
+        one = time.perf_counter() - t_start
+        reps = max(3, min(50, int(12.0 / max(one, 1e-3))))
+        times = []
+        for _ in range(reps):
+            t_start = time.perf_counter()
+            cpu_step()
+            times.append(time.perf_counter() - t_start)
+        times.sort()
+        med = times[len(times) // 2]
+        cpu = {
+            "value": round(step_bytes / med * 1e-9, 2), "unit": "GB/s",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "%d repetitions of the same 2304-token step (median %.1f ms/step) with the "
+                      "PyTorch CPU formulation of the ops (oracle/torch_formulations.py), "
+                      "os.cpu_count()=%d" % (reps, med * 1e3, os.cpu_count()),
+            "ms_per_step": round(med * 1e3, 2),
+        }
+
+    value = step_bytes / (ms_per_step * 1e-3) * 1e-9
+    out = {
+        "metric": "achieved HBM GB/s (% of peak) per fused op at 2304-token hybrid batch",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {
+            "workload": "Llama-3-8B hybrid batch, T=2304 (2048-token prefill chunk at positions "
+                        "4096..6143 + 256 decode tokens): fused_add_rms_norm[2304,4096] -> neox "
+                        "rotary_embedding(q[2304,4096], k[2304,1024], packed qkv, theta=5e5) -> "
+                        "fused_add_rms_norm -> silu_and_mul[2304,28672]",
+            "tokens": T, "bytes_per_step": step_bytes, "buffer_sets": len(sets),
+            "buffer_set_bytes": set_bytes, "cache": "cold (rotating buffer sets)",
+            "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+            "gpu_ms_per_step_events": round(gpu_ms / args.steps, 5),
+            "wall_ms_per_step": round(wall * 1e3 / args.steps, 5),
+            "device": torch.cuda.get_device_name(0),
+        },
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "per_op": per_op,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,151 @@
+/*
+ * sarathi_ops.h -- C ABI of the gfx950 (MI355X) op library that stands in for
+ * Sarathi-Serve's csrc/ ops.
+ *
+ * Conventions, all entry points:
+ *   - plain pointers to DEVICE memory, sizes in ELEMENTS, strides in ELEMENTS;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); the
+ *     call enqueues its kernel(s) on that stream and returns without waiting;
+ *   - nothing is allocated or freed, no global state is mutated, calls are
+ *     re-entrant; the current HIP device must be the one owning the pointers;
+ *   - the return value is 0 on success or a negative SARATHI_ERR_* code; no
+ *     exceptions cross this boundary.  A size of zero tokens is a successful
+ *     no-op.
+ *   - `dtype` is a SARATHI_DTYPE_* code and applies to every floating tensor of
+ *     the call.  16-byte vector paths are chosen when pointers and strides
+ *     allow; otherwise an element-wise path computes the same results.
+ */
+#ifndef SARATHI_OPS_H_
+#define SARATHI_OPS_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SARATHI_OPS_ABI_VERSION 1
+
+/* element types of the floating tensors (csrc/dispatch_utils.h:7-14) */
+#define SARATHI_DTYPE_F32 0
+#define SARATHI_DTYPE_F16 1
+#define SARATHI_DTYPE_BF16 2
+
+/* element types of topk_ids (csrc/dispatch_utils.h:16-24) */
+#define SARATHI_IDTYPE_U8 0
+#define SARATHI_IDTYPE_I8 1
+#define SARATHI_IDTYPE_I16 2
+#define SARATHI_IDTYPE_I32 3
+#define SARATHI_IDTYPE_I64 4
+
+#define SARATHI_OK 0
+#define SARATHI_ERR_INVALID_ARG (-1) /* null pointer, negative size, bad stride */
+#define SARATHI_ERR_UNSUPPORTED (-2) /* unknown dtype code or shape outside limits */
+#define SARATHI_ERR_LAUNCH (-3)      /* the HIP runtime rejected the launch */
+
+/* Largest num_experts accepted by the two MoE routing entry points. */
+#define SARATHI_MOE_MAX_EXPERTS 1024
+
+int sarathi_ops_abi_version(void);
+const char* sarathi_ops_strerror(int code);
+
+/*
+ * Replaces rms_norm(out, input, weight, epsilon): csrc/layernorm.cpp:3-14,
+ * host csrc/layernorm_kernels.cu:39-62.
+ *   out[t,i] = T( T(x[t,i] * rsqrt(mean_i(x[t,:]^2) + eps)) * w[i] ),
+ * sum of squares in fp32.  Rows of `input`/`out` start row_stride elements
+ * apart (the reference assumes hidden_size; pass hidden_size for that).
+ */
+int sarathi_rms_norm(void* out, const void* input, const void* weight, float epsilon,
+                     int64_t num_tokens, int64_t hidden_size, int64_t input_row_stride,
+                     int64_t out_row_stride, int dtype, void* stream);
+
+/*
+ * New entry next to rms_norm; fuses the reference decoder layer's
+ * `hidden = residual + hidden; residual = hidden; hidden = rms_norm(hidden)`
+ * (sarathi/model_executor/models/llama.py:248-252).  In place on both tensors:
+ *   residual <- T(input + residual);  input <- rms_norm(residual).
+ */
+int sarathi_fused_add_rms_norm(void* input, void* residual, const void* weight, float epsilon,
+                               int64_t num_tokens, int64_t hidden_size,
+                               int64_t input_row_stride, int64_t residual_row_stride,
+                               int dtype, void* stream);
+
+/*
+ * Replaces silu_and_mul(out, input): csrc/activation.cpp:3-19, host
+ * csrc/activation_kernels.cu:29-48.  input [num_tokens, 2*d], out
+ * [num_tokens, d]; out = T( T(silu(x)) * y ) with x = input[:, :d],
+ * y = input[:, d:].
+ */
+int sarathi_silu_and_mul(void* out, const void* input, int64_t num_tokens, int64_t d,
+                         int64_t input_row_stride, int64_t out_row_stride, int dtype,
+                         void* stream);
+
+/*
+ * Replace gelu_new(out, input) and gelu_fast(out, input):
+ * csrc/activation.cpp:7-28, csrc/activation_kernels.cu:86-114.
+ * Contiguous [num_tokens, d] in and out.
+ */
+int sarathi_gelu_new(void* out, const void* input, int64_t num_tokens, int64_t d, int dtype,
+                     void* stream);
+int sarathi_gelu_fast(void* out, const void* input, int64_t num_tokens, int64_t d, int dtype,
+                      void* stream);
+
+/*
+ * Replaces rotary_embedding(positions, query, key, head_size, cos_sin_cache,
+ * is_neox): csrc/pos_encoding.cpp:3-16, host csrc/pos_encoding_kernels.cu:80-127.
+ * In place on query [num_tokens, num_heads*head_size] and key
+ * [num_tokens, num_kv_heads*head_size], whose rows start query_stride /
+ * key_stride elements apart (views of a packed qkv buffer are the normal
+ * case).  cos_sin_cache is [max_position, rot_dim] = cos[0:rot/2] || sin[0:rot/2]
+ * per row, in the tensors' dtype; positions are int64 row numbers of that
+ * cache and are not range-checked.  Elements at or above rot_dim in each head
+ * are left untouched.
+ */
+int sarathi_rotary_embedding(const int64_t* positions, void* query, void* key,
+                             const void* cos_sin_cache, int64_t num_tokens, int num_heads,
+                             int num_kv_heads, int head_size, int rot_dim,
+                             int64_t query_stride, int64_t key_stride, int is_neox, int dtype,
+                             void* stream);
+
+/*
+ * Replaces topk_softmax(topk_weights, topk_indices, token_expert_indices,
+ * gating_output): csrc/moe.cpp:3-8, host csrc/moe_topk_softmax_kernels.cu:476-503.
+ * gating_output fp32 [num_tokens, num_experts]; outputs [num_tokens, topk] in
+ * descending probability order, lower expert index first on equal
+ * probabilities; token_expert_indices[t,j] = j*num_tokens + t.  No workspace
+ * is needed for any num_experts in [1, SARATHI_MOE_MAX_EXPERTS]; topk must be
+ * in [1, num_experts].  renormalize = 0 reproduces the reference op (raw
+ * softmax probabilities); renormalize = 1 additionally divides each row's
+ * weights by their sum, which the reference's caller does as a separate
+ * tensor op (sarathi/model_executor/layers/fused_moe/fused_moe.py:371-372).
+ */
+int sarathi_topk_softmax(float* topk_weights, int32_t* topk_indices,
+                         int32_t* token_expert_indices, const float* gating_output,
+                         int64_t num_tokens, int num_experts, int topk, int renormalize,
+                         void* stream);
+
+/*
+ * Replaces moe_align_block_size(topk_ids, num_experts, block_size,
+ * sorted_token_ids, experts_ids, num_tokens_post_pad): csrc/moe.cpp:10-17, host
+ * csrc/moe_align_block_size_kernels.cu:112-135.  Stable counting sort of the
+ * `numel` flat ids by expert, each expert's run padded to a multiple of
+ * block_size.  sorted_token_ids has sorted_len >= numel + E*(block_size-1)
+ * int32 slots, expert_ids has expert_ids_len >= ceil(that / block_size).
+ * Slots of sorted_token_ids that hold no token keep the caller's contents
+ * when fill_pad = 0 (the reference's contract: the caller pre-fills with
+ * numel, fused_moe.py:195) or are set to numel by this call when fill_pad = 1.
+ * expert_ids entries at or above num_tokens_post_pad / block_size are left
+ * untouched.  Ids outside [0, num_experts) are skipped (the reference's
+ * behaviour for them is undefined).
+ */
+int sarathi_moe_align_block_size(const void* topk_ids, int id_dtype, int64_t numel,
+                                 int num_experts, int block_size, int32_t* sorted_token_ids,
+                                 int64_t sorted_len, int32_t* expert_ids,
+                                 int64_t expert_ids_len, int32_t* num_tokens_post_pad,
+                                 int fill_pad, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SARATHI_OPS_H_ */

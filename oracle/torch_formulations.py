@@ -1,0 +1,94 @@
+"""The ops as ordinary CPU PyTorch tensor code.  TEST INFRASTRUCTURE ONLY.
+
+The reference ships no PyTorch fallback for its csrc ops; these are the plain
+tensor-level formulations of what the kernels compute, with the model dtype
+kept wherever the kernels' ``scalar_t`` arithmetic rounds
+(csrc/layernorm_kernels.cu:18-34, csrc/activation_kernels.cu:9-24,
+csrc/pos_encoding_kernels.cu:16-35, csrc/moe_topk_softmax_kernels.cu:261-378,
+csrc/moe_align_block_size_kernels.cu:30-108).  Same positional signatures as
+the reference's pybind modules; results through out-parameters / in place.
+They serve two purposes: an independent check of the C oracle, and the
+multi-threaded CPU baseline timed by the benchmark.
+"""
+import torch
+import torch.nn.functional as F
+
+
+def rms_norm(out, input, weight, epsilon):
+    xf = input.float()
+    var = xf.pow(2).mean(dim=-1, keepdim=True)
+    normed = (xf * torch.rsqrt(var + epsilon)).to(input.dtype)   # first rounding
+    out.copy_(normed * weight)                                    # second rounding
+
+
+def fused_add_rms_norm(input, residual, weight, epsilon):
+    # sarathi/model_executor/models/llama.py:248-252
+    z = residual + input
+    residual.copy_(z)
+    rms_norm(input, z, weight, epsilon)
+
+
+def silu_and_mul(out, input):
+    d = input.shape[-1] // 2
+    out.copy_(F.silu(input[..., :d]) * input[..., d:])
+
+
+def gelu_new(out, input):
+    x = input
+    c = 0.79788456
+    out.copy_(0.5 * x * (1.0 + torch.tanh(c * (x + 0.044715 * x * x * x))))
+
+
+def gelu_fast(out, input):
+    x = input
+    out.copy_(0.5 * x * (1.0 + torch.tanh(x * 0.79788456 * (1.0 + 0.044715 * x * x))))
+
+
+def rotary_embedding(positions, query, key, head_size, cos_sin_cache, is_neox):
+    rot = cos_sin_cache.shape[1]
+    cos, sin = cos_sin_cache[positions].chunk(2, dim=-1)          # [T, rot/2] each
+    cos, sin = cos.unsqueeze(1), sin.unsqueeze(1)
+    for a in (query, key):
+        T = a.shape[0]
+        v = a.view(T, -1, head_size) if a.is_contiguous() else a.unflatten(1, (-1, head_size))
+        r = v[..., :rot]
+        if is_neox:
+            x, y = r[..., : rot // 2], r[..., rot // 2:]
+        else:
+            x, y = r[..., 0::2], r[..., 1::2]
+        nx = x * cos - y * sin        # each tensor op rounds once to the dtype
+        ny = y * cos + x * sin
+        x.copy_(nx)
+        y.copy_(ny)
+
+
+def topk_softmax(topk_weights, topk_indices, token_expert_indices, gating_output):
+    k = topk_weights.shape[-1]
+    T = gating_output.shape[0]
+    p = torch.softmax(gating_output.float(), dim=-1)
+    # a stable descending sort gives "larger value first, lower index on ties"
+    order = torch.sort(p, dim=-1, descending=True, stable=True)
+    topk_weights.copy_(order.values[:, :k])
+    topk_indices.copy_(order.indices[:, :k].to(torch.int32))
+    j = torch.arange(k, dtype=torch.int32).unsqueeze(0)
+    t = torch.arange(T, dtype=torch.int32).unsqueeze(1)
+    token_expert_indices.copy_(j * T + t)
+
+
+def moe_align_block_size(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids,
+                         num_tokens_post_pad):
+    flat = topk_ids.reshape(-1).to(torch.int64)
+    counts = torch.bincount(flat, minlength=num_experts)
+    padded = (counts + block_size - 1) // block_size * block_size
+    cumsum = torch.zeros(num_experts + 1, dtype=torch.int64)
+    cumsum[1:] = torch.cumsum(padded, 0)
+    order = torch.argsort(flat, stable=True)                       # ascending index per expert
+    starts = torch.zeros(num_experts + 1, dtype=torch.int64)
+    starts[1:] = torch.cumsum(counts, 0)
+    sorted_e = flat[order]
+    dest = cumsum[sorted_e] + (torch.arange(flat.numel()) - starts[sorted_e])
+    sorted_token_ids[dest] = order.to(torch.int32)
+    nblk = int(cumsum[-1]) // block_size
+    blk_start = torch.arange(nblk, dtype=torch.int64) * block_size
+    experts_ids[:nblk] = (torch.searchsorted(cumsum, blk_start, right=True) - 1).to(torch.int32)
+    num_tokens_post_pad[0] = int(cumsum[-1])

@@ -1,0 +1,235 @@
+// moe_align_block_size for gfx950: stable counting sort of token->expert ids
+// with every expert's run padded to a multiple of block_size.
+//
+// Replaces csrc/moe_align_block_size_kernels.cu:23-135 of the reference, which
+// runs ONE block of num_experts threads, each walking its shard serially
+// through shared-memory read-modify-writes.  Here one workgroup of W waves
+// (W = 16, or 8 above 512 experts) does the same sort with every lane busy:
+//
+//   1. count   wave w owns a contiguous, ascending chunk of the flat ids and
+//              reads it 64 ids at a time, coalesced.  Inside a 64-id tile the
+//              lanes that hold the same expert find each other with a
+//              bit-serial ballot match (log2(E) ballots), which gives every
+//              lane its rank among equal ids and the group's size; the first
+//              lane of each group adds the size to cnt[w][e] in LDS.
+//   2. scan    per expert, an exclusive scan of cnt[.][e] over the waves (LDS),
+//              then a wave-level prefix scan of the padded totals -> cumsum[].
+//   3. scatter every wave walks its chunk again: slot = cumsum[e] + cnt[w][e]
+//              + rank-in-tile, and the group leader bumps cnt[w][e].  Chunks
+//              are ascending and tiles are visited in order, so the order
+//              inside an expert is ascending token index, exactly the
+//              reference's (stable) order.
+//   4. expert_ids by binary search of cumsum, and (fill_pad) the padding slots
+//              set to numel, the caller-side `fill_` of
+//              sarathi/model_executor/layers/fused_moe/fused_moe.py:195.
+//
+// No atomics, no global scratch, bit-exact by construction.
+#include "vec16.h"
+#include "launch.h"
+
+namespace sarathi_hip {
+
+constexpr int kAlignMaxExperts = SARATHI_MOE_MAX_EXPERTS;  // 1024
+constexpr int kAlignCntInts = 8192;                        // W * E <= 8192
+constexpr int kAlignBatch = 8;                             // tiles loaded ahead per wave
+
+struct TileMatch {
+  int rank;   // lanes below this one holding the same expert
+  int count;  // lanes holding the same expert
+};
+
+// Bit-serial match: after the loop `peers` has a bit for every valid lane of
+// the wave whose expert id equals this lane's.
+SK_DEV TileMatch match_expert(int e, bool valid, int nbits) {
+  unsigned long long peers = __ballot(valid);
+  for (int b = 0; b < nbits; ++b) {
+    const bool bit = (e >> b) & 1;
+    const unsigned long long bal = __ballot(valid && bit);
+    peers &= bit ? bal : ~bal;
+  }
+  const unsigned long long below = (1ull << (threadIdx.x & 63)) - 1ull;
+  TileMatch m;
+  m.rank = __popcll(peers & below);
+  m.count = __popcll(peers);
+  return m;
+}
+
+// ids outside [0, E) become -1 (skipped); done in 64 bits so wide ids cannot wrap into range
+template <typename IdT> SK_DEV int checked_expert(IdT raw, int E) {
+  const int64_t v = (int64_t)raw;
+  return (v >= 0 && v < E) ? (int)v : -1;
+}
+
+template <typename IdT>
+__global__ __launch_bounds__(1024) void moe_align_kernel(
+    const IdT* __restrict__ ids, int64_t numel, int E, int B, int nbits,
+    int32_t* __restrict__ sorted, int64_t sorted_len, int32_t* __restrict__ expert_ids,
+    int64_t expert_ids_len, int32_t* __restrict__ post_pad, int fill_pad) {
+  __shared__ int32_t cnt[kAlignCntInts];            // [W][E]
+  __shared__ int32_t tot[kAlignMaxExperts];         // tokens per expert
+  __shared__ int32_t cumsum[kAlignMaxExperts + 1];  // padded exclusive scan
+
+  const int tid = threadIdx.x;
+  const int nthr = blockDim.x;
+  const int W = nthr >> 6;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+
+  for (int i = tid; i < W * E; i += nthr) cnt[i] = 0;
+  __syncthreads();
+
+  // chunk of this wave: whole tiles, ascending
+  const int64_t tiles_total = (numel + 63) >> 6;
+  const int64_t tiles_per_wave = (tiles_total + W - 1) / W;
+  const int64_t tile_lo = wave * tiles_per_wave;
+  int64_t tile_hi = tile_lo + tiles_per_wave;
+  if (tile_hi > tiles_total) tile_hi = tiles_total;
+  int32_t* my_cnt = cnt + wave * E;
+
+  // ---- 1. count
+  for (int64_t t0 = tile_lo; t0 < tile_hi; t0 += kAlignBatch) {
+    int e[kAlignBatch];
+#pragma unroll
+    for (int u = 0; u < kAlignBatch; ++u) {
+      const int64_t i = ((t0 + u) << 6) + lane;
+      e[u] = (t0 + u < tile_hi && i < numel) ? checked_expert(ids[i], E) : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < kAlignBatch; ++u) {
+      if (t0 + u < tile_hi) {  // wave-uniform
+        const bool valid = e[u] >= 0 && e[u] < E;
+        const TileMatch m = match_expert(e[u], valid, nbits);
+        if (valid && m.rank == 0) my_cnt[e[u]] += m.count;
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- 2. scan over waves per expert, then padded prefix over experts
+  for (int x = tid; x < E; x += nthr) {
+    int run = 0;
+    for (int w = 0; w < W; ++w) {
+      const int c = cnt[w * E + x];
+      cnt[w * E + x] = run;
+      run += c;
+    }
+    tot[x] = run;
+  }
+  __syncthreads();
+  if (wave == 0) {
+    int carry = 0;
+    for (int base = 0; base < E; base += 64) {
+      const int i = base + lane;
+      int x = i < E ? (tot[i] + B - 1) / B * B : 0;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int y = __shfl_up(x, off, 64);
+        if (lane >= off) x += y;
+      }
+      if (i < E) cumsum[i + 1] = carry + x;
+      carry += __shfl(x, 63, 64);
+    }
+    if (lane == 0) {
+      cumsum[0] = 0;
+      *post_pad = carry;
+    }
+  }
+  __syncthreads();
+
+  // ---- 3. scatter
+  for (int64_t t0 = tile_lo; t0 < tile_hi; t0 += kAlignBatch) {
+    int e[kAlignBatch];
+#pragma unroll
+    for (int u = 0; u < kAlignBatch; ++u) {
+      const int64_t i = ((t0 + u) << 6) + lane;
+      e[u] = (t0 + u < tile_hi && i < numel) ? checked_expert(ids[i], E) : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < kAlignBatch; ++u) {
+      if (t0 + u < tile_hi) {
+        const bool valid = e[u] >= 0 && e[u] < E;
+        const TileMatch m = match_expert(e[u], valid, nbits);
+        if (valid) {
+          const int base = my_cnt[e[u]];
+          const int64_t slot = (int64_t)cumsum[e[u]] + base + m.rank;
+          if (slot < sorted_len) sorted[slot] = (int32_t)(((t0 + u) << 6) + lane);
+          if (m.rank == 0) my_cnt[e[u]] = base + m.count;
+        }
+      }
+    }
+  }
+
+  // ---- 4. expert id of every block, padding slots
+  const int total = cumsum[E];
+  const int nblk = total / B;
+  auto expert_of = [&](int pos) {  // largest e with cumsum[e] <= pos, for pos < total
+    int lo = 0, hi = E;            // invariant: cumsum[lo] <= pos < cumsum[hi]
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (cumsum[mid] <= pos) lo = mid; else hi = mid;
+    }
+    return lo;
+  };
+  for (int b = tid; b < nblk; b += nthr)
+    if (b < expert_ids_len) expert_ids[b] = expert_of(b * B);
+  if (fill_pad) {
+    const int32_t pad = (int32_t)numel;
+    for (int64_t i = tid; i < sorted_len; i += nthr) {
+      bool is_pad = true;
+      if (i < total) {
+        const int x = expert_of((int)i);
+        is_pad = (int)i - cumsum[x] >= tot[x];
+      }
+      if (is_pad) sorted[i] = pad;
+    }
+  }
+}
+
+template <typename IdT>
+static int launch_align(const void* ids, int64_t numel, int E, int B, int32_t* sorted,
+                        int64_t sorted_len, int32_t* expert_ids, int64_t expert_ids_len,
+                        int32_t* post_pad, int fill_pad, hipStream_t st) {
+  int nbits = 0;
+  while ((1 << nbits) < E) ++nbits;
+  const int threads = E <= 512 ? 1024 : 512;
+  hipLaunchKernelGGL((moe_align_kernel<IdT>), dim3(1), dim3(threads), 0, st,
+                     reinterpret_cast<const IdT*>(ids), numel, E, B, nbits, sorted, sorted_len,
+                     expert_ids, expert_ids_len, post_pad, fill_pad);
+  return launch_status();
+}
+
+}  // namespace sarathi_hip
+
+extern "C" int sarathi_moe_align_block_size(const void* topk_ids, int id_dtype, int64_t numel,
+                                            int num_experts, int block_size,
+                                            int32_t* sorted_token_ids, int64_t sorted_len,
+                                            int32_t* expert_ids, int64_t expert_ids_len,
+                                            int32_t* num_tokens_post_pad, int fill_pad,
+                                            void* stream) {
+  using namespace sarathi_hip;
+  if (!sorted_token_ids || !expert_ids || !num_tokens_post_pad) return SARATHI_ERR_INVALID_ARG;
+  if (numel < 0 || (numel > 0 && !topk_ids) || num_experts <= 0 || block_size <= 0 ||
+      sorted_len < 0 || expert_ids_len < 0)
+    return SARATHI_ERR_INVALID_ARG;
+  if (num_experts > kAlignMaxExperts) return SARATHI_ERR_UNSUPPORTED;
+  // worst case of num_tokens_post_pad: every non-empty expert wastes block_size - 1 slots
+  const int64_t nonempty_max = numel < num_experts ? numel : num_experts;
+  const int64_t worst = numel + nonempty_max * ((int64_t)block_size - 1);
+  if (worst > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
+  if (sorted_len < worst || expert_ids_len * (int64_t)block_size < worst)
+    return SARATHI_ERR_INVALID_ARG;
+  hipStream_t st = (hipStream_t)stream;
+#define SK_ALIGN(T)                                                                      \
+  return launch_align<T>(topk_ids, numel, num_experts, block_size, sorted_token_ids,     \
+                         sorted_len, expert_ids, expert_ids_len, num_tokens_post_pad,    \
+                         fill_pad, st)
+  switch (id_dtype) {
+    case SARATHI_IDTYPE_U8: SK_ALIGN(uint8_t);
+    case SARATHI_IDTYPE_I8: SK_ALIGN(int8_t);
+    case SARATHI_IDTYPE_I16: SK_ALIGN(int16_t);
+    case SARATHI_IDTYPE_I32: SK_ALIGN(int32_t);
+    case SARATHI_IDTYPE_I64: SK_ALIGN(int64_t);
+    default: return SARATHI_ERR_UNSUPPORTED;
+  }
+#undef SK_ALIGN
+}

@@ -1,0 +1,190 @@
+// rms_norm and fused_add_rms_norm for gfx950.
+//
+// Replaces csrc/layernorm_kernels.cu:11-62 of the reference (one 1024-thread
+// block per token, 2-byte loads, the row read twice, a two-level shared-memory
+// reduction).  Here one 64-lane wave owns one token row and keeps it in
+// registers: the row is read from HBM exactly once with 16-byte loads that are
+// all issued before the first use, the sum of squares is folded inside the wave
+// with DPP, and the normalised row is written with 16-byte stores.  No LDS and
+// no barrier.  A block is four independent waves (four rows).
+//
+// Arithmetic (rounding points as in the reference):
+//   ss = sum f32(x)^2 ; s = rsqrt(ss / H + eps)
+//   out = T( f32(T(f32(x) * s)) * f32(w) )
+// and for the fused op first z = T(f32(x) + f32(r)), residual <- z, x := z.
+#include "vec16.h"
+#include "launch.h"
+
+namespace sarathi_hip {
+
+constexpr int kRmsWavesPerBlock = 4;
+
+// VPL = 16-byte vectors held per lane; the row has nvec <= 64 * VPL vectors.
+template <int DT, int VPL, bool FUSED>
+__global__ __launch_bounds__(64 * kRmsWavesPerBlock) void rms_norm_wave_kernel(
+    void* out,        // FUSED: the `input` tensor, updated in place
+    void* in_or_res,  // FUSED: the residual tensor, updated in place
+    const void* __restrict__ weight, float eps, int64_t num_tokens, int nvec, float hidden_f,
+    int64_t out_stride_vec, int64_t in_stride_vec) {
+  constexpr int N = VecElems<DT>::value;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * kRmsWavesPerBlock + (threadIdx.x >> 6);
+  if (row >= num_tokens) return;  // wave-uniform
+
+  const int64_t in_base = row * in_stride_vec;
+  const int64_t out_base = row * out_stride_vec;
+
+  u32x4 raw[VPL];
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    int c = lane + 64 * j;
+    raw[j] = c < nvec ? load16_stream(in_or_res, in_base + c) : (u32x4){0, 0, 0, 0};
+  }
+  if constexpr (FUSED) {
+    u32x4 hid[VPL];
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      int c = lane + 64 * j;
+      hid[j] = c < nvec ? load16_stream(out, out_base + c) : (u32x4){0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      Vec<DT> a, b;
+      a.unpack(raw[j]);
+      b.unpack(hid[j]);
+#pragma unroll
+      for (int i = 0; i < N; ++i) a.f[i] = b.f[i] + a.f[i];
+      raw[j] = a.pack();  // z, rounded to the dtype
+      int c = lane + 64 * j;
+      if (c < nvec) store16_stream(in_or_res, in_base + c, raw[j]);
+    }
+  }
+
+  // weight vectors are shared by every row and stay cache resident; fetch them
+  // now so their latency overlaps the reduction
+  u32x4 wraw[VPL];
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    int c = lane + 64 * j;
+    wraw[j] = c < nvec ? load16(weight, c) : (u32x4){0, 0, 0, 0};
+  }
+
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    Vec<DT> a;
+    a.unpack(raw[j]);
+#pragma unroll
+    for (int i = 0; i < N; ++i) ss = __builtin_fmaf(a.f[i], a.f[i], ss);
+  }
+  ss = wave64_sum(ss);
+  const float s = __builtin_amdgcn_rsqf(ss / hidden_f + eps);
+
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    int c = lane + 64 * j;
+    if (c < nvec) {
+      Vec<DT> a, w;
+      a.unpack(raw[j]);
+      w.unpack(wraw[j]);
+#pragma unroll
+      for (int i = 0; i < N; ++i) a.f[i] = rnd<DT>(a.f[i] * s) * w.f[i];
+      store16_stream(out, out_base + c, a.pack());
+    }
+  }
+}
+
+// Any shape / alignment: one 256-thread block per row, element-wise accesses,
+// the row re-read from cache for the second pass.
+template <int DT, bool FUSED>
+__global__ __launch_bounds__(256) void rms_norm_generic_kernel(
+    void* out, void* in_or_res, const void* __restrict__ weight, float eps, int hidden,
+    float hidden_f, int64_t out_stride, int64_t in_stride) {
+  __shared__ float partial[4];
+  const int64_t row = blockIdx.x;
+  const int64_t ib = row * in_stride, ob = row * out_stride;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += 256) {
+    float x = load_elem<DT>(in_or_res, ib + i);
+    if constexpr (FUSED) {
+      x = rnd<DT>(load_elem<DT>(out, ob + i) + x);
+      store_elem<DT>(in_or_res, ib + i, x);
+    }
+    ss = __builtin_fmaf(x, x, ss);
+  }
+  ss = wave64_sum(ss);
+  if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = ss;
+  __syncthreads();  // also orders the residual stores above before the re-read below
+  ss = (partial[0] + partial[1]) + (partial[2] + partial[3]);
+  const float s = __builtin_amdgcn_rsqf(ss / hidden_f + eps);
+  for (int i = threadIdx.x; i < hidden; i += 256) {
+    float x = load_elem<DT>(in_or_res, ib + i);
+    store_elem<DT>(out, ob + i, rnd<DT>(x * s) * load_elem<DT>(weight, i));
+  }
+}
+
+template <int DT, bool FUSED>
+static int launch_rms(void* out, void* in, const void* w, float eps, int64_t T, int64_t H,
+                      int64_t out_stride, int64_t in_stride, hipStream_t st) {
+  constexpr int N = VecElems<DT>::value;
+  const float hidden_f = (float)H;
+  const bool vec_ok = (H % N == 0) && (out_stride % N == 0) && (in_stride % N == 0) &&
+                      aligned16(out) && aligned16(in) && aligned16(w) && (H / N) <= 64 * 16;
+  if (!vec_ok) {
+    if (T > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((rms_norm_generic_kernel<DT, FUSED>), dim3((unsigned)T), dim3(256), 0, st,
+                       out, in, w, eps, (int)H, hidden_f, out_stride, in_stride);
+    return launch_status();
+  }
+  const int nvec = (int)(H / N);
+  const int64_t blocks = (T + kRmsWavesPerBlock - 1) / kRmsWavesPerBlock;
+  if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
+  dim3 grid((unsigned)blocks), block(64 * kRmsWavesPerBlock);
+  const int vpl = (nvec + 63) / 64;
+#define SK_RMS_CASE(V)                                                                        \
+  hipLaunchKernelGGL((rms_norm_wave_kernel<DT, V, FUSED>), grid, block, 0, st, out, in, w, eps, \
+                     T, nvec, hidden_f, out_stride / N, in_stride / N)
+  if (vpl <= 1) SK_RMS_CASE(1);
+  else if (vpl <= 2) SK_RMS_CASE(2);
+  else if (vpl <= 4) SK_RMS_CASE(4);
+  else if (vpl <= 8) SK_RMS_CASE(8);
+  else SK_RMS_CASE(16);
+#undef SK_RMS_CASE
+  return launch_status();
+}
+
+template <bool FUSED>
+static int dispatch_rms(void* out, void* in, const void* w, float eps, int64_t T, int64_t H,
+                        int64_t out_stride, int64_t in_stride, int dtype, void* stream) {
+  if (!out || !in || !w) return SARATHI_ERR_INVALID_ARG;
+  if (T < 0 || H <= 0 || out_stride < H || in_stride < H) return SARATHI_ERR_INVALID_ARG;
+  if (H > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
+  if (T == 0) return SARATHI_OK;
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case kBF16: return launch_rms<kBF16, FUSED>(out, in, w, eps, T, H, out_stride, in_stride, st);
+    case kF16: return launch_rms<kF16, FUSED>(out, in, w, eps, T, H, out_stride, in_stride, st);
+    case kF32: return launch_rms<kF32, FUSED>(out, in, w, eps, T, H, out_stride, in_stride, st);
+    default: return SARATHI_ERR_UNSUPPORTED;
+  }
+}
+
+}  // namespace sarathi_hip
+
+extern "C" int sarathi_rms_norm(void* out, const void* input, const void* weight, float epsilon,
+                                int64_t num_tokens, int64_t hidden_size,
+                                int64_t input_row_stride, int64_t out_row_stride, int dtype,
+                                void* stream) {
+  return sarathi_hip::dispatch_rms<false>(out, const_cast<void*>(input), weight, epsilon,
+                                          num_tokens, hidden_size, out_row_stride,
+                                          input_row_stride, dtype, stream);
+}
+
+extern "C" int sarathi_fused_add_rms_norm(void* input, void* residual, const void* weight,
+                                          float epsilon, int64_t num_tokens, int64_t hidden_size,
+                                          int64_t input_row_stride, int64_t residual_row_stride,
+                                          int dtype, void* stream) {
+  return sarathi_hip::dispatch_rms<true>(input, residual, weight, epsilon, num_tokens,
+                                         hidden_size, input_row_stride, residual_row_stride,
+                                         dtype, stream);
+}

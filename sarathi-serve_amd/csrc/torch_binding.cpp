@@ -1,0 +1,298 @@
+// PyTorch-ROCm front end of the op library: a pybind11 module whose functions
+// have the names and positional signatures of the reference's four extension
+// modules (csrc/layernorm.cpp:9, csrc/activation.cpp:15-27, csrc/pos_encoding.cpp:11,
+// csrc/moe.cpp:19-27), plus fused_add_rms_norm and two fused MoE variants.
+//
+// This layer only (a) checks what the reference leaves unchecked: device, dtype,
+// rank, inner contiguity; (b) makes the tensors' device current and looks up
+// torch's current HIP stream for it; (c) forwards raw pointers, sizes and
+// strides to the C ABI of include/sarathi_ops.h and turns a non-zero status
+// into a RuntimeError.  It never allocates, copies or synchronises.
+#include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
+#include <torch/extension.h>
+
+#include "../../include/sarathi_ops.h"
+
+namespace {
+
+int dtype_code(const torch::Tensor& t, const char* op) {
+  switch (t.scalar_type()) {
+    case at::ScalarType::Float: return SARATHI_DTYPE_F32;
+    case at::ScalarType::Half: return SARATHI_DTYPE_F16;
+    case at::ScalarType::BFloat16: return SARATHI_DTYPE_BF16;
+    default: TORCH_CHECK(false, op, ": expected a float32, float16 or bfloat16 tensor, got ",
+                         t.scalar_type());
+  }
+  return -1;
+}
+
+int id_dtype_code(const torch::Tensor& t) {
+  switch (t.scalar_type()) {
+    case at::ScalarType::Byte: return SARATHI_IDTYPE_U8;
+    case at::ScalarType::Char: return SARATHI_IDTYPE_I8;
+    case at::ScalarType::Short: return SARATHI_IDTYPE_I16;
+    case at::ScalarType::Int: return SARATHI_IDTYPE_I32;
+    case at::ScalarType::Long: return SARATHI_IDTYPE_I64;
+    default: TORCH_CHECK(false, "moe_align_block_size: topk_ids must be an integer tensor, got ",
+                         t.scalar_type());
+  }
+  return -1;
+}
+
+void check_gpu(const torch::Tensor& t, const torch::Tensor& like, const char* op,
+               const char* name) {
+  TORCH_CHECK(t.is_cuda(), op, ": ", name, " must live on the GPU");
+  TORCH_CHECK(t.device() == like.device(), op, ": ", name, " is on ", t.device(),
+              " but the first tensor is on ", like.device());
+}
+
+// Makes `dev` the current HIP device for the scope and yields torch's current
+// stream on it.
+struct LaunchScope {
+  int prev = -1;
+  int dev;
+  void* stream;
+  explicit LaunchScope(const torch::Tensor& t) : dev(t.device().index()) {
+    TORCH_CHECK(hipGetDevice(&prev) == hipSuccess, "hipGetDevice failed");
+    if (prev != dev) TORCH_CHECK(hipSetDevice(dev) == hipSuccess, "hipSetDevice failed");
+    stream = c10::hip::getCurrentHIPStream(static_cast<c10::DeviceIndex>(dev)).stream();
+  }
+  ~LaunchScope() {
+    if (prev >= 0 && prev != dev) (void)hipSetDevice(prev);
+  }
+};
+
+void raise_on(int status, const char* op) {
+  TORCH_CHECK(status == SARATHI_OK, op, " failed: ", sarathi_ops_strerror(status), " (code ",
+              status, ")");
+}
+
+// ---- layernorm_ops -----------------------------------------------------------
+
+void rms_norm(torch::Tensor& out, torch::Tensor& input, torch::Tensor& weight, double epsilon) {
+  const char* op = "rms_norm";
+  check_gpu(input, input, op, "input");
+  check_gpu(out, input, op, "out");
+  check_gpu(weight, input, op, "weight");
+  TORCH_CHECK(input.dim() == 2 && out.dim() == 2, op, ": input and out must be [num_tokens, hidden]");
+  TORCH_CHECK(out.sizes() == input.sizes(), op, ": out and input shapes differ");
+  TORCH_CHECK(out.scalar_type() == input.scalar_type() &&
+                  weight.scalar_type() == input.scalar_type(),
+              op, ": out, input and weight must share a dtype");
+  TORCH_CHECK(weight.dim() == 1 && weight.size(0) == input.size(1) && weight.is_contiguous(), op,
+              ": weight must be a contiguous [hidden] vector");
+  TORCH_CHECK(input.stride(1) == 1 && out.stride(1) == 1, op, ": rows must be contiguous");
+  LaunchScope scope(input);
+  raise_on(sarathi_rms_norm(out.data_ptr(), input.data_ptr(), weight.data_ptr(), (float)epsilon,
+                            input.size(0), input.size(1), input.stride(0), out.stride(0),
+                            dtype_code(input, op), scope.stream),
+           op);
+}
+
+void fused_add_rms_norm(torch::Tensor& input, torch::Tensor& residual, torch::Tensor& weight,
+                        double epsilon) {
+  const char* op = "fused_add_rms_norm";
+  check_gpu(input, input, op, "input");
+  check_gpu(residual, input, op, "residual");
+  check_gpu(weight, input, op, "weight");
+  TORCH_CHECK(input.dim() == 2, op, ": input must be [num_tokens, hidden]");
+  TORCH_CHECK(residual.sizes() == input.sizes(), op, ": residual and input shapes differ");
+  TORCH_CHECK(residual.scalar_type() == input.scalar_type() &&
+                  weight.scalar_type() == input.scalar_type(),
+              op, ": input, residual and weight must share a dtype");
+  TORCH_CHECK(weight.dim() == 1 && weight.size(0) == input.size(1) && weight.is_contiguous(), op,
+              ": weight must be a contiguous [hidden] vector");
+  TORCH_CHECK(input.stride(1) == 1 && residual.stride(1) == 1, op, ": rows must be contiguous");
+  TORCH_CHECK(input.data_ptr() != residual.data_ptr(), op, ": input and residual must not alias");
+  LaunchScope scope(input);
+  raise_on(sarathi_fused_add_rms_norm(input.data_ptr(), residual.data_ptr(), weight.data_ptr(),
+                                      (float)epsilon, input.size(0), input.size(1),
+                                      input.stride(0), residual.stride(0), dtype_code(input, op),
+                                      scope.stream),
+           op);
+}
+
+// ---- activation_ops ----------------------------------------------------------
+
+void silu_and_mul(torch::Tensor& out, torch::Tensor& input) {
+  const char* op = "silu_and_mul";
+  check_gpu(input, input, op, "input");
+  check_gpu(out, input, op, "out");
+  TORCH_CHECK(input.dim() == 2 && out.dim() == 2, op, ": input [num_tokens, 2*d], out [num_tokens, d]");
+  TORCH_CHECK(input.size(1) % 2 == 0 && out.size(1) * 2 == input.size(1) &&
+                  out.size(0) == input.size(0),
+              op, ": out must be [num_tokens, input.size(1) / 2]");
+  TORCH_CHECK(out.scalar_type() == input.scalar_type(), op, ": out and input must share a dtype");
+  TORCH_CHECK(input.stride(1) == 1 && out.stride(1) == 1, op, ": rows must be contiguous");
+  LaunchScope scope(input);
+  raise_on(sarathi_silu_and_mul(out.data_ptr(), input.data_ptr(), input.size(0), out.size(1),
+                                input.stride(0), out.stride(0), dtype_code(input, op),
+                                scope.stream),
+           op);
+}
+
+template <bool FAST>
+void gelu_impl(torch::Tensor& out, torch::Tensor& input) {
+  const char* op = FAST ? "gelu_fast" : "gelu_new";
+  check_gpu(input, input, op, "input");
+  check_gpu(out, input, op, "out");
+  TORCH_CHECK(input.dim() == 2 && out.sizes() == input.sizes(), op,
+              ": input and out must both be [num_tokens, d]");
+  TORCH_CHECK(out.scalar_type() == input.scalar_type(), op, ": out and input must share a dtype");
+  TORCH_CHECK(input.is_contiguous() && out.is_contiguous(), op, ": tensors must be contiguous");
+  LaunchScope scope(input);
+  auto fn = FAST ? sarathi_gelu_fast : sarathi_gelu_new;
+  raise_on(fn(out.data_ptr(), input.data_ptr(), input.size(0), input.size(1),
+              dtype_code(input, op), scope.stream),
+           op);
+}
+void gelu_new(torch::Tensor& out, torch::Tensor& input) { gelu_impl<false>(out, input); }
+void gelu_fast(torch::Tensor& out, torch::Tensor& input) { gelu_impl<true>(out, input); }
+
+// ---- pos_encoding_ops --------------------------------------------------------
+
+void rotary_embedding(torch::Tensor& positions, torch::Tensor& query, torch::Tensor& key,
+                      int64_t head_size, torch::Tensor& cos_sin_cache, bool is_neox) {
+  const char* op = "rotary_embedding";
+  check_gpu(query, query, op, "query");
+  check_gpu(key, query, op, "key");
+  check_gpu(positions, query, op, "positions");
+  check_gpu(cos_sin_cache, query, op, "cos_sin_cache");
+  TORCH_CHECK(positions.scalar_type() == at::ScalarType::Long && positions.dim() == 1 &&
+                  positions.is_contiguous(),
+              op, ": positions must be a contiguous int64 [num_tokens] tensor");
+  TORCH_CHECK(query.dim() == 2 && key.dim() == 2, op, ": query and key must be 2-D");
+  TORCH_CHECK(query.size(0) == positions.size(0) && key.size(0) == positions.size(0), op,
+              ": query, key and positions disagree on num_tokens");
+  TORCH_CHECK(key.scalar_type() == query.scalar_type() &&
+                  cos_sin_cache.scalar_type() == query.scalar_type(),
+              op, ": query, key and cos_sin_cache must share a dtype");
+  TORCH_CHECK(head_size > 0 && query.size(1) % head_size == 0 && key.size(1) % head_size == 0, op,
+              ": row widths must be multiples of head_size");
+  TORCH_CHECK(cos_sin_cache.dim() == 2 && cos_sin_cache.is_contiguous(), op,
+              ": cos_sin_cache must be a contiguous [max_position, rot_dim] tensor");
+  TORCH_CHECK(query.stride(1) == 1 && key.stride(1) == 1, op, ": rows must be contiguous");
+  const int64_t rot_dim = cos_sin_cache.size(1);
+  TORCH_CHECK(rot_dim % 2 == 0 && rot_dim <= head_size, op, ": rot_dim must be even and <= head_size");
+  LaunchScope scope(query);
+  raise_on(sarathi_rotary_embedding(positions.data_ptr<int64_t>(), query.data_ptr(), key.data_ptr(),
+                                    cos_sin_cache.data_ptr(), query.size(0),
+                                    (int)(query.size(1) / head_size),
+                                    (int)(key.size(1) / head_size), (int)head_size, (int)rot_dim,
+                                    query.stride(0), key.stride(0), is_neox ? 1 : 0,
+                                    dtype_code(query, op), scope.stream),
+           op);
+}
+
+// ---- moe_ops -----------------------------------------------------------------
+
+void topk_softmax_impl(torch::Tensor& topk_weights, torch::Tensor& topk_indices,
+                       torch::Tensor& token_expert_indices, torch::Tensor& gating_output,
+                       bool renormalize, const char* op) {
+  check_gpu(gating_output, gating_output, op, "gating_output");
+  check_gpu(topk_weights, gating_output, op, "topk_weights");
+  check_gpu(topk_indices, gating_output, op, "topk_indices");
+  check_gpu(token_expert_indices, gating_output, op, "token_expert_indices");
+  TORCH_CHECK(gating_output.scalar_type() == at::ScalarType::Float &&
+                  topk_weights.scalar_type() == at::ScalarType::Float,
+              op, ": gating_output and topk_weights must be float32");
+  TORCH_CHECK(topk_indices.scalar_type() == at::ScalarType::Int &&
+                  token_expert_indices.scalar_type() == at::ScalarType::Int,
+              op, ": topk_indices and token_expert_indices must be int32");
+  TORCH_CHECK(gating_output.dim() >= 1 && gating_output.is_contiguous() &&
+                  topk_weights.is_contiguous() && topk_indices.is_contiguous() &&
+                  token_expert_indices.is_contiguous(),
+              op, ": tensors must be contiguous");
+  const int64_t num_experts = gating_output.size(-1);
+  TORCH_CHECK(num_experts > 0, op, ": gating_output has no experts");
+  const int64_t num_tokens = gating_output.numel() / num_experts;
+  const int64_t topk = topk_weights.size(-1);
+  TORCH_CHECK(topk_weights.numel() == num_tokens * topk && topk_indices.numel() == num_tokens * topk &&
+                  token_expert_indices.numel() == num_tokens * topk,
+              op, ": outputs must be [num_tokens, topk]");
+  LaunchScope scope(gating_output);
+  raise_on(sarathi_topk_softmax(topk_weights.data_ptr<float>(), topk_indices.data_ptr<int32_t>(),
+                                token_expert_indices.data_ptr<int32_t>(),
+                                gating_output.data_ptr<float>(), num_tokens, (int)num_experts,
+                                (int)topk, renormalize ? 1 : 0, scope.stream),
+           op);
+}
+
+void topk_softmax(torch::Tensor& topk_weights, torch::Tensor& topk_indices,
+                  torch::Tensor& token_expert_indices, torch::Tensor& gating_output) {
+  topk_softmax_impl(topk_weights, topk_indices, token_expert_indices, gating_output, false,
+                    "topk_softmax");
+}
+
+void topk_softmax_renorm(torch::Tensor& topk_weights, torch::Tensor& topk_indices,
+                         torch::Tensor& token_expert_indices, torch::Tensor& gating_output) {
+  topk_softmax_impl(topk_weights, topk_indices, token_expert_indices, gating_output, true,
+                    "topk_softmax_renorm");
+}
+
+void moe_align_impl(torch::Tensor& topk_ids, int64_t num_experts, int64_t block_size,
+                    torch::Tensor& sorted_token_ids, torch::Tensor& experts_ids,
+                    torch::Tensor& num_tokens_post_pad, bool fill_pad, const char* op) {
+  check_gpu(topk_ids, topk_ids, op, "topk_ids");
+  check_gpu(sorted_token_ids, topk_ids, op, "sorted_token_ids");
+  check_gpu(experts_ids, topk_ids, op, "experts_ids");
+  check_gpu(num_tokens_post_pad, topk_ids, op, "num_tokens_post_pad");
+  TORCH_CHECK(sorted_token_ids.scalar_type() == at::ScalarType::Int &&
+                  experts_ids.scalar_type() == at::ScalarType::Int &&
+                  num_tokens_post_pad.scalar_type() == at::ScalarType::Int,
+              op, ": sorted_token_ids, experts_ids and num_tokens_post_pad must be int32");
+  TORCH_CHECK(topk_ids.is_contiguous() && sorted_token_ids.is_contiguous() &&
+                  experts_ids.is_contiguous() && num_tokens_post_pad.numel() >= 1,
+              op, ": tensors must be contiguous");
+  TORCH_CHECK(num_experts > 0 && num_experts <= INT32_MAX && block_size > 0 &&
+                  block_size <= INT32_MAX,
+              op, ": num_experts and block_size must be positive");
+  LaunchScope scope(topk_ids);
+  raise_on(sarathi_moe_align_block_size(
+               topk_ids.data_ptr(), id_dtype_code(topk_ids), topk_ids.numel(), (int)num_experts,
+               (int)block_size, sorted_token_ids.data_ptr<int32_t>(), sorted_token_ids.numel(),
+               experts_ids.data_ptr<int32_t>(), experts_ids.numel(),
+               num_tokens_post_pad.data_ptr<int32_t>(), fill_pad ? 1 : 0, scope.stream),
+           op);
+}
+
+void moe_align_block_size(torch::Tensor topk_ids, int64_t num_experts, int64_t block_size,
+                          torch::Tensor sorted_token_ids, torch::Tensor experts_ids,
+                          torch::Tensor num_tokens_post_pad) {
+  moe_align_impl(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids,
+                 num_tokens_post_pad, false, "moe_align_block_size");
+}
+
+void moe_align_block_size_filled(torch::Tensor topk_ids, int64_t num_experts, int64_t block_size,
+                                 torch::Tensor sorted_token_ids, torch::Tensor experts_ids,
+                                 torch::Tensor num_tokens_post_pad) {
+  moe_align_impl(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids,
+                 num_tokens_post_pad, true, "moe_align_block_size_filled");
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.doc() = "gfx950 HIP implementation of Sarathi-Serve's csrc op library";
+  m.def("abi_version", &sarathi_ops_abi_version);
+  // layernorm_ops
+  m.def("rms_norm", &rms_norm, "out = rms_norm(input) * weight");
+  m.def("fused_add_rms_norm", &fused_add_rms_norm,
+        "residual += input; input = rms_norm(residual) * weight (both in place)");
+  // activation_ops
+  m.def("silu_and_mul", &silu_and_mul, "out = silu(input[:, :d]) * input[:, d:]");
+  m.def("gelu_new", &gelu_new, "GPT-2 tanh GELU");
+  m.def("gelu_fast", &gelu_fast, "approximate tanh GELU");
+  // pos_encoding_ops
+  m.def("rotary_embedding", &rotary_embedding,
+        "in-place GPT-NeoX / GPT-J rotary embedding of query and key");
+  // moe_ops
+  m.def("topk_softmax", &topk_softmax, "softmax over experts + top-k (raw probabilities)");
+  m.def("topk_softmax_renorm", &topk_softmax_renorm,
+        "topk_softmax with the k weights of each token renormalised to sum to 1");
+  m.def("moe_align_block_size", &moe_align_block_size,
+        "stable sort of token ids by expert, runs padded to block_size");
+  m.def("moe_align_block_size_filled", &moe_align_block_size_filled,
+        "moe_align_block_size that also writes the padding value into unused slots");
+}

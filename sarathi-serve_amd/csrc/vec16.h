@@ -1,0 +1,153 @@
+// 16-byte vector access and dtype conversion helpers for gfx950 kernels.
+//
+// Every dense kernel in this library moves data as one 16-byte global access
+// per lane (global_load_dwordx4 / global_store_dwordx4): 8 bf16 or fp16
+// elements, or 4 fp32 elements.  Arithmetic is always fp32; `rnd<DT>()` is the
+// "cast to the tensor dtype and widen again" step that the reference's
+// scalar_t arithmetic performs between operations.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sarathi_hip {
+
+enum : int { kF32 = 0, kF16 = 1, kBF16 = 2 };
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+#define SK_DEV __device__ __forceinline__
+
+template <int DT> struct ElemBytes { static constexpr int value = 2; };
+template <> struct ElemBytes<kF32> { static constexpr int value = 4; };
+
+// elements per 16-byte vector
+template <int DT> struct VecElems { static constexpr int value = 16 / ElemBytes<DT>::value; };
+
+// ---- packed 32-bit word <-> two floats -------------------------------------
+
+template <int DT> SK_DEV f32x2 unpack2(uint32_t w);
+template <> SK_DEV f32x2 unpack2<kBF16>(uint32_t w) {
+  f32x2 r;
+  r.x = __builtin_bit_cast(float, w << 16);
+  r.y = __builtin_bit_cast(float, w & 0xffff0000u);
+  return r;
+}
+template <> SK_DEV f32x2 unpack2<kF16>(uint32_t w) {
+  return __builtin_convertvector(__builtin_bit_cast(f16x2, w), f32x2);
+}
+
+// round-to-nearest-even pack (v_cvt_pk_bf16_f32 / v_cvt_f16_f32 on gfx950)
+template <int DT> SK_DEV uint32_t pack2(float a, float b);
+template <> SK_DEV uint32_t pack2<kBF16>(float a, float b) {
+  f32x2 v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+template <> SK_DEV uint32_t pack2<kF16>(float a, float b) {
+  f32x2 v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
+
+// Round a float to the tensor dtype and widen again.
+template <int DT> SK_DEV float rnd(float f);
+template <> SK_DEV float rnd<kF32>(float f) { return f; }
+template <> SK_DEV float rnd<kBF16>(float f) { return (float)(__bf16)f; }
+template <> SK_DEV float rnd<kF16>(float f) { return (float)(_Float16)f; }
+
+// ---- a 16-byte vector as an array of floats --------------------------------
+
+template <int DT> struct Vec {
+  static constexpr int N = VecElems<DT>::value;
+  float f[N];
+
+  SK_DEV void unpack(u32x4 v) {
+    if constexpr (DT == kF32) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) f[i] = __builtin_bit_cast(float, v[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        f32x2 p = unpack2<DT>(v[i]);
+        f[2 * i] = p.x;
+        f[2 * i + 1] = p.y;
+      }
+    }
+  }
+  // rounds to the dtype
+  SK_DEV u32x4 pack() const {
+    u32x4 v;
+    if constexpr (DT == kF32) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = __builtin_bit_cast(uint32_t, f[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = pack2<DT>(f[2 * i], f[2 * i + 1]);
+    }
+    return v;
+  }
+};
+
+// ---- global memory ---------------------------------------------------------
+
+// Streaming (read-once / write-once) 16-byte accesses carry the `nt` hint so
+// they do not displace the reusable rows (weights, cos/sin cache) in L2.
+SK_DEV u32x4 load16_stream(const void* base, int64_t vec_index) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(base) + vec_index);
+}
+SK_DEV void store16_stream(void* base, int64_t vec_index, u32x4 v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(base) + vec_index);
+}
+SK_DEV u32x4 load16(const void* base, int64_t vec_index) {
+  return reinterpret_cast<const u32x4*>(base)[vec_index];
+}
+SK_DEV void store16(void* base, int64_t vec_index, u32x4 v) {
+  reinterpret_cast<u32x4*>(base)[vec_index] = v;
+}
+
+// Element-wise accessors for the unaligned fallback paths.
+template <int DT> SK_DEV float load_elem(const void* base, int64_t i) {
+  if constexpr (DT == kF32) return reinterpret_cast<const float*>(base)[i];
+  else if constexpr (DT == kBF16)
+    return __builtin_bit_cast(float, (uint32_t)reinterpret_cast<const uint16_t*>(base)[i] << 16);
+  else return (float)reinterpret_cast<const _Float16*>(base)[i];
+}
+template <int DT> SK_DEV void store_elem(void* base, int64_t i, float v) {
+  if constexpr (DT == kF32) reinterpret_cast<float*>(base)[i] = v;
+  else if constexpr (DT == kBF16) reinterpret_cast<__bf16*>(base)[i] = (__bf16)v;
+  else reinterpret_cast<_Float16*>(base)[i] = (_Float16)v;
+}
+
+// ---- wave64 reductions -------------------------------------------------------
+
+// Adds `v` across the 64 lanes of a wave; every lane returns the total.
+// Four DPP steps fold each row of 16 lanes (quad swaps, then the half-row and
+// row mirrors, which are valid folds because each group being mirrored is
+// already uniform), then the four row totals are read as scalars and added.
+template <int CTRL> SK_DEV float dpp_fold_add(float x) {
+  int y = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false);
+  return x + __builtin_bit_cast(float, y);
+}
+SK_DEV float wave64_sum(float v) {
+  v = dpp_fold_add<0xB1>(v);   // quad_perm [1,0,3,2]
+  v = dpp_fold_add<0x4E>(v);   // quad_perm [2,3,0,1]
+  v = dpp_fold_add<0x141>(v);  // row_half_mirror
+  v = dpp_fold_add<0x140>(v);  // row_mirror
+  int b = __builtin_bit_cast(int, v);
+  float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0));
+  float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+  float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32));
+  float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+  return (r0 + r1) + (r2 + r3);
+}
+
+SK_DEV float wave64_max(float v) {
+#pragma unroll
+  for (int m = 32; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
+  return v;
+}
+
+}  // namespace sarathi_hip

@@ -1,0 +1,16 @@
+"""Counterpart of the reference's ``sarathi.moe_ops`` (csrc/moe.cpp:19-28).
+
+``topk_softmax_renorm`` and ``moe_align_block_size_filled`` are fused variants:
+the first also performs the caller-side renormalisation of
+sarathi/model_executor/layers/fused_moe/fused_moe.py:371-372, the second the
+caller-side ``sorted_ids.fill_(numel)`` of fused_moe.py:195.
+"""
+from ._ext import C as _C
+
+topk_softmax = _C.topk_softmax
+moe_align_block_size = _C.moe_align_block_size
+topk_softmax_renorm = _C.topk_softmax_renorm
+moe_align_block_size_filled = _C.moe_align_block_size_filled
+
+__all__ = ["topk_softmax", "moe_align_block_size", "topk_softmax_renorm",
+           "moe_align_block_size_filled"]

@@ -1,0 +1,61 @@
+"""Seeded inputs of the benchmark configurations and comparison helpers shared by the tests.
+
+Inputs are always drawn on the CPU in fp32 from a seeded generator and then cast, so the oracle
+(CPU) and the HIP kernels (GPU copy of the same tensor) see identical bits.
+"""
+import torch
+
+THETA_LLAMA3 = 500000.0
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def randn(shape, g, dtype=torch.bfloat16, mean=0.0, std=1.0):
+    return (torch.randn(shape, generator=g, dtype=torch.float32) * std + mean).to(dtype)
+
+
+def hybrid_positions(num_tokens, prefill_len, g, prefill_start=4096, max_pos=8192):
+    """One prefill chunk at consecutive positions followed by decode tokens at random positions
+    (prefill tokens come first in a hybrid batch: sarathi/model_executor/model_runner.py:76-104)."""
+    pre = torch.arange(prefill_start, prefill_start + prefill_len, dtype=torch.int64)
+    dec = torch.randint(1, max_pos, (num_tokens - prefill_len,), generator=g, dtype=torch.int64)
+    return torch.cat((pre, dec))
+
+
+def cos_sin_cache(max_pos, rot_dim, theta, dtype):
+    """cos || sin table as sarathi/model_executor/layers/rotary_embedding.py:55-84 builds it,
+    computed on the CPU in fp32 and cast to the model dtype."""
+    inv_freq = 1.0 / (theta ** (torch.arange(0, rot_dim, 2, dtype=torch.float32) / rot_dim))
+    t = torch.arange(max_pos, dtype=torch.float32)
+    freqs = torch.outer(t, inv_freq)
+    return torch.cat((freqs.cos(), freqs.sin()), dim=-1).to(dtype)
+
+
+def ulp_of(t):
+    """Spacing of the tensor's dtype at each element's magnitude (as float32)."""
+    mant = {torch.bfloat16: 7, torch.float16: 10, torch.float32: 23}[t.dtype]
+    mag = t.float().abs().clamp_min(2.0 ** -126)
+    return torch.exp2(torch.floor(torch.log2(mag)) - mant)
+
+
+def assert_close_dtype(got, want, atol=1e-2, rtol=1e-2, max_ulps=1, max_mismatch_frac=5e-3):
+    """The stated tolerance (|got-want| <= atol + rtol*|want|, i.e. torch.allclose semantics with
+    atol = rtol = 1e-2) plus the much tighter bound the kernels actually meet: no element is off
+    by more than `max_ulps` units in the last place of the dtype and only a small fraction is off
+    at all."""
+    got, want = got.cpu(), want.cpu()
+    assert got.shape == want.shape and got.dtype == want.dtype
+    g, w = got.float(), want.float()
+    assert torch.isfinite(g).all() == torch.isfinite(w).all()
+    diff = (g - w).abs()
+    assert bool((diff <= atol + rtol * w.abs()).all()), (
+        "outside tolerance: max abs %.4g" % diff.max().item())
+    bad = diff > 0
+    frac = bad.float().mean().item()
+    if bad.any():
+        ulps = (diff / torch.maximum(ulp_of(got), ulp_of(want)))[bad].max().item()
+        assert ulps <= max_ulps + 1e-3, "max error %.2f ulp" % ulps
+    assert frac <= max_mismatch_frac, "mismatching fraction %.3g" % frac
+    return frac

@@ -1,0 +1,227 @@
+"""GPU parity of the dense layer ops (rms_norm, fused_add_rms_norm, silu_and_mul, gelu_*,
+rotary_embedding) against the CPU oracle on identical seeded inputs.
+
+Every call goes through the shipped op namespaces, i.e. pybind front end -> C ABI -> HIP kernel.
+Tolerance for 16-bit outputs: |got - want| <= 1e-2 + 1e-2 * |want| (atol = rtol = 1e-2); the
+helper additionally requires every mismatch to be a single unit in the last place.  rotary_embedding
+and the residual output of fused_add_rms_norm have no transcendental and must be bit-exact.
+"""
+import pytest
+import torch
+
+from helpers import (THETA_LLAMA3, assert_close_dtype, cos_sin_cache, gen, hybrid_positions, randn)
+from oracle import c_oracle
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.bfloat16, torch.float16, torch.float32]
+
+
+def _tol(dtype):
+    # fp32 results differ from the oracle only through exp / rsqrt / reduction order
+    return dict(atol=1e-2, rtol=1e-2, max_ulps=1 if dtype != torch.float32 else 64,
+                max_mismatch_frac=5e-3 if dtype != torch.float32 else 1.0)
+
+
+# ---------------------------------------------------------------- rms_norm
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,H", [(512, 4096), (37, 8192), (5, 1024), (3, 512), (7, 320), (2, 16384),
+                                 (4, 100), (1, 8)])
+def test_rms_norm_matches_oracle(ops, dev, dtype, T, H):
+    g = gen(100 + H)
+    x = randn((T, H), g, dtype)
+    w = randn((H,), g, dtype, mean=1.0, std=0.1)
+    want = torch.empty_like(x)
+    c_oracle.rms_norm(want, x, w, 1e-5)
+    got = torch.empty_like(x, device=dev)
+    ops.layernorm_ops.rms_norm(got, x.to(dev), w.to(dev), 1e-5)
+    assert_close_dtype(got, want, **_tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,H", [(512, 4096), (37, 8192), (5, 1024), (7, 320), (2, 16384), (4, 100)])
+def test_fused_add_rms_norm_matches_oracle(ops, dev, dtype, T, H):
+    # (512, 4096) bf16 is the benchmark's CPU-path configuration
+    g = gen(0)
+    x = randn((T, H), g, dtype)
+    r = randn((T, H), g, dtype)
+    w = randn((H,), g, dtype, mean=1.0, std=0.1)
+    wx, wr = x.clone(), r.clone()
+    c_oracle.fused_add_rms_norm(wx, wr, w, 1e-5)
+    gx, gr = x.to(dev), r.to(dev)
+    ops.layernorm_ops.fused_add_rms_norm(gx, gr, w.to(dev), 1e-5)
+    assert torch.equal(gr.cpu(), wr), "residual = T(x + r) must be bit-exact"
+    assert_close_dtype(gx, wx, **_tol(dtype))
+
+
+def test_fused_add_equals_add_then_norm_bitwise(ops, dev):
+    """fused(x, r) == (r' = x + r in bf16; rms_norm(r')) bit for bit, using the library's own
+    rms_norm: the fusion changes traffic, not arithmetic."""
+    g = gen(3)
+    T, H = 2304, 4096
+    x, r = randn((T, H), g).to(dev), randn((T, H), g).to(dev)
+    w = randn((H,), g, mean=1.0, std=0.1).to(dev)
+    z = r + x
+    want = torch.empty_like(z)
+    ops.layernorm_ops.rms_norm(want, z, w, 1e-5)
+    ops.layernorm_ops.fused_add_rms_norm(x, r, w, 1e-5)
+    assert torch.equal(r, z) and torch.equal(x, want)
+
+
+def test_rms_norm_row_strides(ops, dev):
+    """Rows may be views with a row stride larger than the width."""
+    g = gen(4)
+    big = randn((64, 3 * 1024), g).to(dev)
+    x = big[:, 1024:2048]
+    w = randn((1024,), g, mean=1.0, std=0.1).to(dev)
+    out_big = torch.zeros((64, 2048), dtype=torch.bfloat16, device=dev)
+    out = out_big[:, :1024]
+    ops.layernorm_ops.rms_norm(out, x, w, 1e-6)
+    want = torch.empty((64, 1024), dtype=torch.bfloat16)
+    c_oracle.rms_norm(want, x.cpu().contiguous(), w.cpu(), 1e-6)
+    assert_close_dtype(out.contiguous(), want)
+    assert bool((out_big[:, 1024:] == 0).all())
+
+
+def test_rms_norm_full_size_properties(ops, dev):
+    """Llama-3-70B shape [4608, 8192]: scale invariance in the input (x -> 2x leaves the output
+    unchanged up to eps), and rows are independent (a permutation of rows permutes the output)."""
+    g = gen(5)
+    T, H = 4608, 8192
+    x = randn((T, H), g).to(dev)
+    w = randn((H,), g, mean=1.0, std=0.1).to(dev)
+    a, b = torch.empty_like(x), torch.empty_like(x)
+    ops.layernorm_ops.rms_norm(a, x, w, 0.0)
+    ops.layernorm_ops.rms_norm(b, x * 2, w, 0.0)        # exact doubling in bf16
+    assert torch.equal(a, b)
+    perm = torch.randperm(T, generator=g).to(dev)
+    c = torch.empty_like(x)
+    ops.layernorm_ops.rms_norm(c, x[perm].contiguous(), w, 0.0)
+    assert torch.equal(c, a[perm])
+
+
+# -------------------------------------------------------------- activation
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,d", [(64, 14336), (9, 4096), (5, 1000), (3, 7), (1, 8)])
+def test_silu_and_mul_matches_oracle(ops, dev, dtype, T, d):
+    g = gen(2)
+    x = randn((T, 2 * d), g, dtype, std=2.0)
+    want = torch.empty((T, d), dtype=dtype)
+    c_oracle.silu_and_mul(want, x)
+    got = torch.empty((T, d), dtype=dtype, device=dev)
+    ops.activation_ops.silu_and_mul(got, x.to(dev))
+    assert_close_dtype(got, want, **_tol(dtype))
+
+
+def test_silu_and_mul_special_values(ops, dev):
+    xs = torch.tensor([0.0, -0.0, 1.0, -1.0, 30.0, -30.0, 100.0, -100.0, 1e4, -1e4,
+                       float("inf"), 1e-3, -1e-3, 88.0, -88.0, -104.0], dtype=torch.float32)
+    x = torch.cat((xs, torch.ones_like(xs))).bfloat16().reshape(1, -1)
+    want = torch.empty((1, xs.numel()), dtype=torch.bfloat16)
+    c_oracle.silu_and_mul(want, x)
+    got = torch.empty_like(want, device=dev)
+    ops.activation_ops.silu_and_mul(got, x.to(dev))
+    assert_close_dtype(got, want, max_mismatch_frac=1.0)
+
+
+def test_silu_and_mul_full_size_properties(ops, dev):
+    """Llama-3-8B MLP shape [2304, 2*14336]: y = 1 reduces the op to silu (library routine), and
+    the op is odd-linear in y: f(x, -y) = -f(x, y) exactly."""
+    g = gen(6)
+    T, d = 2304, 14336
+    x = randn((T, 2 * d), g).to(dev)
+    out = torch.empty((T, d), dtype=torch.bfloat16, device=dev)
+    ops.activation_ops.silu_and_mul(out, x)
+    neg = x.clone()
+    neg[:, d:] = -neg[:, d:]
+    out2 = torch.empty_like(out)
+    ops.activation_ops.silu_and_mul(out2, neg)
+    assert torch.equal(out2, -out)
+    ones = x.clone()
+    ones[:, d:] = 1.0
+    ops.activation_ops.silu_and_mul(out2, ones)
+    ref = torch.nn.functional.silu(x[:, :d].float()).bfloat16()
+    assert_close_dtype(out2, ref, max_mismatch_frac=5e-3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["gelu_new", "gelu_fast"])
+@pytest.mark.parametrize("T,d", [(33, 4096), (5, 1001), (1, 3)])
+def test_gelu_matches_oracle(ops, dev, dtype, name, T, d):
+    g = gen(7)
+    x = randn((T, d), g, dtype, std=2.0)
+    want = torch.empty_like(x)
+    getattr(c_oracle, name)(want, x)
+    got = torch.empty_like(x, device=dev)
+    getattr(ops.activation_ops, name)(got, x.to(dev))
+    # the chains of dtype roundings amplify a last-place difference in tanh by up to 2 ulp
+    tol = _tol(dtype)
+    tol["max_ulps"] = max(tol["max_ulps"], 2)
+    tol["max_mismatch_frac"] = max(tol["max_mismatch_frac"], 2e-2)
+    assert_close_dtype(got, want, **tol)
+
+
+# ------------------------------------------------------------------ rotary
+
+def _rope_case(ops, dev, dtype, T, nq, nkv, D, R, is_neox, packed, seed=1, prefill=None):
+    g = gen(seed)
+    cache = cos_sin_cache(8192, R, THETA_LLAMA3, dtype)
+    pos = hybrid_positions(T, prefill if prefill is not None else (T * 8) // 9, g)
+    if packed:
+        qkv = randn((T, (nq + 2 * nkv) * D), g, dtype)
+        want = qkv.clone()
+        wq, wk, _ = want.split([nq * D, nkv * D, nkv * D], dim=-1)
+        c_oracle.rotary_embedding(pos, wq, wk, D, cache, is_neox)
+        got = qkv.to(dev)
+        gq, gk, _ = got.split([nq * D, nkv * D, nkv * D], dim=-1)
+        ops.pos_encoding_ops.rotary_embedding(pos.to(dev), gq, gk, D, cache.to(dev), is_neox)
+        return got.cpu(), want
+    q, k = randn((T, nq * D), g, dtype), randn((T, nkv * D), g, dtype)
+    wq, wk = q.clone(), k.clone()
+    c_oracle.rotary_embedding(pos, wq, wk, D, cache, is_neox)
+    gq, gk = q.to(dev), k.to(dev)
+    ops.pos_encoding_ops.rotary_embedding(pos.to(dev), gq, gk, D, cache.to(dev), is_neox)
+    return torch.cat((gq.cpu(), gk.cpu()), -1), torch.cat((wq, wk), -1)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("is_neox", [True, False])
+@pytest.mark.parametrize("packed", [False, True])
+def test_rope_llama3_8b_hybrid_batch_bit_exact(ops, dev, dtype, is_neox, packed):
+    """The benchmark configuration: T = 2304 = 2048 prefill + 256 decode, 32 q / 8 kv heads of 128."""
+    got, want = _rope_case(ops, dev, dtype, 2304, 32, 8, 128, 128, is_neox, packed, prefill=2048)
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("is_neox", [True, False])
+@pytest.mark.parametrize("T,nq,nkv,D,R", [
+    (4608 // 8, 64, 8, 128, 128),   # Llama-3-70B head counts
+    (17, 4, 4, 64, 64),
+    (9, 8, 2, 128, 64),             # partial rotary: elements >= rot_dim untouched
+    (5, 3, 1, 96, 32),
+    (3, 2, 2, 80, 20),              # rot_dim/2 not a multiple of the vector width -> element path
+    (1, 1, 1, 256, 256),
+    (11, 160, 8, 128, 128),         # more heads than one pass of the block covers
+])
+def test_rope_shapes_bit_exact(ops, dev, T, nq, nkv, D, R, is_neox):
+    for packed in (False, True):
+        got, want = _rope_case(ops, dev, torch.bfloat16, T, nq, nkv, D, R, is_neox, packed, seed=T)
+        assert torch.equal(got, want)
+
+
+def test_rope_position_zero_is_identity_and_norm_preserved(ops, dev):
+    g = gen(8)
+    T, nq, nkv, D = 256, 32, 8, 128
+    cache = cos_sin_cache(8192, D, THETA_LLAMA3, torch.float32)
+    q, k = randn((T, nq * D), g, torch.float32), randn((T, nkv * D), g, torch.float32)
+    gq, gk = q.to(dev), k.to(dev)
+    ops.pos_encoding_ops.rotary_embedding(torch.zeros(T, dtype=torch.int64, device=dev), gq, gk, D,
+                                          cache.to(dev), True)
+    assert torch.equal(gq.cpu(), q) and torch.equal(gk.cpu(), k)     # cos = 1, sin = 0
+    pos = hybrid_positions(T, 128, g)
+    ops.pos_encoding_ops.rotary_embedding(pos.to(dev), gq, gk, D, cache.to(dev), True)
+    n0 = q.view(T, nq, 2, D // 2).pow(2).sum(2)
+    n1 = gq.cpu().view(T, nq, 2, D // 2).pow(2).sum(2)
+    assert torch.allclose(n0, n1, rtol=1e-5, atol=1e-6)              # rotations keep |(x, y)|

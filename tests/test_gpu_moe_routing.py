@@ -1,0 +1,194 @@
+"""GPU parity of MoE routing (topk_softmax, moe_align_block_size) against the CPU oracle.
+
+Indices, sorted_token_ids, expert_ids (valid prefix) and num_tokens_post_pad must be bit-exact;
+softmax weights are compared to 1e-6 (the device and host expf differ in the last place).
+"""
+import json
+import os
+
+import pytest
+import torch
+
+from helpers import gen
+from oracle import c_oracle
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                      "moe_align_block_size_vectors.json")
+
+
+def _topk_gpu(ops, dev, gating, k, renorm=False):
+    T = gating.shape[0]
+    w = torch.empty((T, k), dtype=torch.float32, device=dev)
+    idx = torch.empty((T, k), dtype=torch.int32, device=dev)
+    src = torch.empty((T, k), dtype=torch.int32, device=dev)
+    fn = ops.moe_ops.topk_softmax_renorm if renorm else ops.moe_ops.topk_softmax
+    fn(w, idx, src, gating.to(dev))
+    return w.cpu(), idx.cpu(), src.cpu()
+
+
+def _topk_oracle(gating, k):
+    T = gating.shape[0]
+    w = torch.empty((T, k), dtype=torch.float32)
+    idx = torch.empty((T, k), dtype=torch.int32)
+    src = torch.empty((T, k), dtype=torch.int32)
+    c_oracle.topk_softmax(w, idx, src, gating)
+    return w, idx, src
+
+
+def _assert_separated(gating, k):
+    """Indices are only well defined across expf implementations when the k+1 largest logits of
+    every row are distinct by more than rounding noise; assert it for the seeded input."""
+    top = torch.sort(gating, dim=-1, descending=True).values[:, : k + 1]
+    if top.shape[1] > 1:
+        assert (top[:, :-1] - top[:, 1:]).min().item() > 1e-6
+
+
+@pytest.mark.parametrize("E,k", [(8, 2), (1, 1), (2, 1), (2, 2), (4, 2), (16, 4), (32, 5), (64, 6),
+                                 (128, 8), (256, 8), (8, 8), (60, 4), (6, 2), (100, 3), (384, 8),
+                                 (1000, 2)])
+def test_topk_softmax_matches_oracle(ops, dev, E, k):
+    g = gen(3)
+    T = 4096 if E == 8 else 515
+    gating = torch.randn((T, E), generator=g, dtype=torch.float32)
+    _assert_separated(gating, min(k, E - 1))
+    ww, wi, ws = _topk_oracle(gating, k)
+    gw, gi, gs = _topk_gpu(ops, dev, gating, k)
+    assert torch.equal(gi, wi)
+    assert torch.equal(gs, ws)
+    assert torch.allclose(gw, ww, rtol=0, atol=1e-6)
+
+
+def test_topk_softmax_ties_and_collapsed_probabilities(ops, dev):
+    """Equal logits: lower expert index first.  Logits so far below the maximum that their
+    probabilities are exactly 0 tie at 0 and are also taken in index order (the reference compares
+    probabilities, not logits)."""
+    rows = torch.tensor([
+        [1.0] * 8,
+        [0.0, 5.0, 5.0, 0.0, 5.0, 0.0, 0.0, 0.0],
+        [0.0, -300.0, -200.0, -250.0, -400.0, -210.0, -220.0, -230.0],
+        [-1e4, -1e4, 3.0, -1e4, -1e4, -1e4, -1e4, -2e4],
+    ], dtype=torch.float32)
+    ww, wi, ws = _topk_oracle(rows, 3)
+    gw, gi, gs = _topk_gpu(ops, dev, rows, 3)
+    assert wi.tolist() == [[0, 1, 2], [1, 2, 4], [0, 1, 2], [2, 0, 1]]
+    assert torch.equal(gi, wi) and torch.equal(gs, ws)
+    assert torch.allclose(gw, ww, rtol=0, atol=1e-6)
+
+
+def test_topk_softmax_renorm_equals_caller_side_division(ops, dev):
+    g = gen(3)
+    gating = torch.randn((4096, 8), generator=g, dtype=torch.float32)
+    w, i, _ = _topk_gpu(ops, dev, gating, 2)
+    wr, ir, _ = _topk_gpu(ops, dev, gating, 2, renorm=True)
+    assert torch.equal(i, ir)
+    assert torch.equal(wr, w / w.sum(dim=-1, keepdim=True))   # same fp32 add and divide
+
+
+def _align_bufs(numel, E, B, device, fill=True):
+    n = numel + E * (B - 1)
+    s = torch.empty((n,), dtype=torch.int32, device=device)
+    s.fill_(numel if fill else -7)
+    e = torch.full(((n + B - 1) // B,), -1, dtype=torch.int32, device=device)
+    p = torch.full((1,), -1, dtype=torch.int32, device=device)
+    return s, e, p
+
+
+def _align_both(ops, dev, ids, E, B, filled=False):
+    ws, we, wp = _align_bufs(ids.numel(), E, B, "cpu")
+    c_oracle.moe_align_block_size(ids, E, B, ws, we, wp)
+    gs, ge, gp = _align_bufs(ids.numel(), E, B, dev, fill=not filled)
+    fn = ops.moe_ops.moe_align_block_size_filled if filled else ops.moe_ops.moe_align_block_size
+    fn(ids.to(dev), E, B, gs, ge, gp)
+    return (gs.cpu(), ge.cpu(), gp.cpu()), (ws, we, wp)
+
+
+def _check_align(got, want, B):
+    (gs, ge, gp), (ws, we, wp) = got, want
+    assert torch.equal(gp, wp)
+    assert torch.equal(gs, ws)                       # full length, padding slots included
+    nblk = int(wp.item()) // B
+    assert torch.equal(ge[:nblk], we[:nblk])
+    assert bool((ge[nblk:] == -1).all())             # entries past the valid prefix untouched
+
+
+def test_moe_align_reference_vectors(ops, dev):
+    with open(GOLDEN) as f:
+        vectors = json.load(f)["vectors"]
+    for v in vectors:
+        ids = torch.tensor(v["topk_ids"], dtype=torch.int32)
+        E, B = v["num_experts"], v["block_size"]
+        for filled in (False, True):
+            gs, ge, gp = _align_bufs(ids.numel(), E, B, dev, fill=not filled)
+            fn = (ops.moe_ops.moe_align_block_size_filled if filled
+                  else ops.moe_ops.moe_align_block_size)
+            fn(ids.to(dev), E, B, gs, ge, gp)
+            n = v["num_tokens_post_pad"]
+            assert gp.item() == n
+            assert gs.cpu()[:n].tolist() == v["sorted_token_ids_prefix"]
+            assert bool((gs.cpu()[n:] == ids.numel()).all())
+            assert ge.cpu()[: n // B].tolist() == v["expert_ids_prefix"]
+
+
+@pytest.mark.parametrize("filled", [False, True])
+@pytest.mark.parametrize("T,k,E,B", [(4096, 2, 8, 64), (4096, 2, 8, 16), (4096, 2, 8, 128),
+                                     (1, 1, 8, 64), (7, 2, 8, 32), (63, 1, 4, 4), (64, 1, 4, 4),
+                                     (65, 3, 16, 1), (1000, 6, 64, 16), (3000, 8, 256, 32),
+                                     (500, 4, 1000, 8), (70000, 2, 8, 64), (16384, 4, 60, 128)])
+def test_moe_align_matches_oracle(ops, dev, T, k, E, B, filled):
+    g = gen(T + E)
+    ids = torch.randint(0, E, (T, k), generator=g, dtype=torch.int32)
+    _check_align(*_align_both(ops, dev, ids, E, B, filled), B)
+
+
+def test_moe_align_from_config4_topk(ops, dev):
+    """Mixtral-shaped routing end to end: logits [4096, 8] -> top-2 -> align with block 64."""
+    g = gen(3)
+    gating = torch.randn((4096, 8), generator=g, dtype=torch.float32)
+    _, ids, _ = _topk_gpu(ops, dev, gating, 2)
+    _, want_ids, _ = _topk_oracle(gating, 2)
+    assert torch.equal(ids, want_ids)
+    got, want = _align_both(ops, dev, ids, 8, 64)
+    _check_align(got, want, 64)
+    assert got[0].numel() == 8696 and got[1].numel() == 136
+
+
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64])
+def test_moe_align_id_dtypes(ops, dev, dtype):
+    g = gen(11)
+    ids = torch.randint(0, 100, (777, 2), generator=g, dtype=torch.int32).to(dtype)
+    _check_align(*_align_both(ops, dev, ids, 100, 16), 16)
+
+
+def test_moe_align_skewed_and_empty(ops, dev):
+    # everything on one expert; some experts empty; empty input
+    ids = torch.full((5000,), 3, dtype=torch.int32)
+    _check_align(*_align_both(ops, dev, ids, 8, 64), 64)
+    ids = torch.tensor([7, 7, 0, 7, 0], dtype=torch.int32)
+    _check_align(*_align_both(ops, dev, ids, 8, 4, filled=True), 4)
+    ids = torch.empty((0,), dtype=torch.int32)
+    _check_align(*_align_both(ops, dev, ids, 8, 4, filled=True), 4)
+
+
+def test_moe_align_invariants_large(ops, dev):
+    """64K tokens x top-2 (the largest chunk the reference's caller passes, fused_moe.py:459):
+    non-padding entries are a permutation of 0..numel-1, each block holds one expert's tokens in
+    ascending order, post_pad = sum ceil(cnt/B)*B."""
+    g = gen(12)
+    T, k, E, B = 65536, 2, 8, 64
+    ids = torch.randint(0, E, (T, k), generator=g, dtype=torch.int32)
+    gs, ge, gp = _align_bufs(T * k, E, B, dev, fill=False)
+    ops.moe_ops.moe_align_block_size_filled(ids.to(dev), E, B, gs, ge, gp)
+    gs, ge, n = gs.cpu(), ge.cpu(), int(gp.item())
+    flat = ids.reshape(-1)
+    cnt = torch.bincount(flat.long(), minlength=E)
+    assert n == int(((cnt + B - 1) // B * B).sum()) and n % B == 0
+    real = gs[:n][gs[:n] != T * k]
+    assert torch.equal(torch.sort(real).values, torch.arange(T * k, dtype=torch.int32))
+    blocks = gs[:n].view(-1, B)
+    for b in range(blocks.shape[0]):
+        row = blocks[b][blocks[b] != T * k].long()
+        assert bool((flat[row] == ge[b]).all())
+        assert bool((row[1:] > row[:-1]).all())
+    assert bool((gs[n:] == T * k).all())
