@@ -2,11 +2,14 @@
 //
 // Replaces csrc/activation_kernels.cu:8-114 of the reference (one block per
 // token, 2-byte __ldg loads, a per-thread loop over the row).  These are pure
-// streaming ops, so the whole design is about bytes in flight: a thread owns
-// one 16-byte column slot of ROWS consecutive token rows, issues all of its
-// 16-byte loads before the first use, and writes 16-byte stores.  A block is
-// 256 lanes wide (4 KiB contiguous per row segment), the grid is
-// (row groups) x (column chunks), i.e. thousands of blocks for 256 CUs.
+// streaming ops.  What measured fastest on MI355X is the opposite of a fat
+// persistent kernel: one 64-lane workgroup per 1 KiB segment of a row, every
+// lane doing exactly one 16-byte load per input stream and one 16-byte store,
+// with workgroup ids running along the row first and then down the rows, so
+// that the workgroups in flight at any moment sweep memory linearly (the same
+// kernel with row-major workgroup order is ~12 % slower, and every extra vector
+// per lane costs a few percent).  Row bases live in scalar registers as buffer
+// resources; ragged row ends are clipped by the hardware range check.
 //
 // Arithmetic, rounding points as in the reference (fp32 math, T = tensor dtype):
 //   silu_and_mul: out = T( f32(T( x / (1 + exp(-x)) )) * y )
@@ -19,7 +22,9 @@
 
 namespace sarathi_hip {
 
-constexpr int kActBlock = 256;
+constexpr int kActBlock = 256;   // element-wise fallback kernels
+constexpr int kRowSeg = 64;      // lanes per workgroup of the streaming kernels
+constexpr int kMaxGridY = 65535;
 
 SK_DEV float silu_f32(float x) {
   // x * sigmoid(x) = x / (1 + 2^(-x * log2 e))
@@ -36,36 +41,25 @@ SK_DEV float tanh_f32(float u) {
 
 // ---- silu_and_mul ------------------------------------------------------------
 
-template <int DT, int ROWS>
-__global__ __launch_bounds__(kActBlock) void silu_and_mul_kernel(
-    void* __restrict__ out, const void* __restrict__ in, int64_t num_tokens, int nvec_d,
-    int64_t in_stride_vec, int64_t out_stride_vec) {
+template <int DT>
+__global__ __launch_bounds__(kRowSeg) void silu_and_mul_kernel(
+    void* __restrict__ out, const void* __restrict__ in, uint32_t half_row_bytes,
+    int64_t in_stride_bytes, int64_t out_stride_bytes) {
   constexpr int N = VecElems<DT>::value;
-  const int col = blockIdx.y * kActBlock + threadIdx.x;
-  if (col >= nvec_d) return;
-  const int64_t row0 = (int64_t)blockIdx.x * ROWS;
-
-  u32x4 xr[ROWS], yr[ROWS];
+  const int64_t row = (int64_t)blockIdx.z * kMaxGridY + blockIdx.y;
+  const rsrc_t rx = make_rsrc(reinterpret_cast<const char*>(in) + row * in_stride_bytes,
+                              half_row_bytes);
+  const rsrc_t ry = make_rsrc(
+      reinterpret_cast<const char*>(in) + row * in_stride_bytes + half_row_bytes, half_row_bytes);
+  const rsrc_t ro = make_rsrc(reinterpret_cast<char*>(out) + row * out_stride_bytes,
+                              half_row_bytes);
+  const uint32_t off = (blockIdx.x * kRowSeg + threadIdx.x) * 16u;
+  Vec<DT> x, y;
+  x.unpack(buf_load16<kStreamLoad>(rx, off));
+  y.unpack(buf_load16<kStreamLoad>(ry, off));
 #pragma unroll
-  for (int r = 0; r < ROWS; ++r) {
-    const int64_t row = row0 + r;
-    if (row < num_tokens) {
-      xr[r] = load16_stream(in, row * in_stride_vec + col);
-      yr[r] = load16_stream(in, row * in_stride_vec + nvec_d + col);
-    }
-  }
-#pragma unroll
-  for (int r = 0; r < ROWS; ++r) {
-    const int64_t row = row0 + r;
-    if (row < num_tokens) {
-      Vec<DT> x, y;
-      x.unpack(xr[r]);
-      y.unpack(yr[r]);
-#pragma unroll
-      for (int i = 0; i < N; ++i) x.f[i] = rnd<DT>(silu_f32(x.f[i])) * y.f[i];
-      store16_stream(out, row * out_stride_vec + col, x.pack());
-    }
-  }
+  for (int i = 0; i < N; ++i) x.f[i] = rnd<DT>(silu_f32(x.f[i])) * y.f[i];
+  buf_store16<kStreamStore>(ro, off, x.pack());
 }
 
 template <int DT>
@@ -84,9 +78,9 @@ template <int DT>
 static int launch_silu(void* out, const void* in, int64_t T, int64_t d, int64_t in_stride,
                        int64_t out_stride, hipStream_t st) {
   constexpr int N = VecElems<DT>::value;
-  constexpr int ROWS = 4;
+  constexpr int EB = ElemBytes<DT>::value;
   const bool vec_ok = (d % N == 0) && (in_stride % N == 0) && (out_stride % N == 0) &&
-                      aligned16(out) && aligned16(in);
+                      aligned16(out) && aligned16(in) && d * EB <= 0x7fffffffLL;
   if (T > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
   if (!vec_ok) {
     hipLaunchKernelGGL((silu_and_mul_generic_kernel<DT>), dim3((unsigned)T), dim3(kActBlock), 0,
@@ -94,11 +88,23 @@ static int launch_silu(void* out, const void* in, int64_t T, int64_t d, int64_t 
     return launch_status();
   }
   const int64_t nvec_d = d / N;
-  const int64_t chunks = (nvec_d + kActBlock - 1) / kActBlock;
-  if (chunks > 65535) return SARATHI_ERR_UNSUPPORTED;
-  dim3 grid((unsigned)((T + ROWS - 1) / ROWS), (unsigned)chunks);
-  hipLaunchKernelGGL((silu_and_mul_kernel<DT, ROWS>), grid, dim3(kActBlock), 0, st, out, in, T,
-                     (int)nvec_d, in_stride / N, out_stride / N);
+  const int64_t segs = (nvec_d + kRowSeg - 1) / kRowSeg;
+  // rows above 65535 spill into grid.z; the last z-slice may run past T, so launch it apart
+  const int64_t full_z = T / kMaxGridY, rem = T % kMaxGridY;
+  const char* inb = reinterpret_cast<const char*>(in);
+  char* outb = reinterpret_cast<char*>(out);
+  if (full_z > 0) {
+    hipLaunchKernelGGL((silu_and_mul_kernel<DT>), dim3((unsigned)segs, kMaxGridY, (unsigned)full_z),
+                       dim3(kRowSeg), 0, st, out, in, (uint32_t)(d * EB), in_stride * EB,
+                       out_stride * EB);
+  }
+  if (rem > 0) {
+    const int64_t r0 = full_z * kMaxGridY;
+    hipLaunchKernelGGL((silu_and_mul_kernel<DT>), dim3((unsigned)segs, (unsigned)rem, 1),
+                       dim3(kRowSeg), 0, st, outb + r0 * out_stride * EB,
+                       inb + r0 * in_stride * EB, (uint32_t)(d * EB), in_stride * EB,
+                       out_stride * EB);
+  }
   return launch_status();
 }
 
@@ -122,37 +128,33 @@ template <int DT> SK_DEV float gelu_fast_elem(float x) {
   return rnd<DT>(0.5f * x) * rnd<DT>(1.0f + t);
 }
 
-// Flat element-wise kernel over n16 16-byte vectors plus a scalar tail.
-template <int DT, bool FAST, int UNROLL>
-__global__ __launch_bounds__(kActBlock) void gelu_kernel(void* __restrict__ out,
-                                                         const void* __restrict__ in,
-                                                         int64_t n16, int64_t numel) {
+// Flat element-wise kernel: the tensor is cut into spans of kGeluSpan bytes (one
+// buffer resource each, grid.y), a workgroup handles 1 KiB of a span.  Elements
+// past the last whole vector go through the scalar tail in workgroup (0, 0).
+constexpr uint32_t kGeluSpan = 1u << 30;
+
+template <int DT, bool FAST>
+__global__ __launch_bounds__(kRowSeg) void gelu_kernel(void* __restrict__ out,
+                                                       const void* __restrict__ in,
+                                                       int64_t vec_bytes, int64_t numel) {
   constexpr int N = VecElems<DT>::value;
-  const int64_t base = ((int64_t)blockIdx.x * UNROLL) * kActBlock + threadIdx.x;
-  u32x4 raw[UNROLL];
+  const int64_t span0 = (int64_t)blockIdx.y * kGeluSpan;
+  const int64_t left = vec_bytes - span0;
+  const uint32_t span_bytes = left < (int64_t)kGeluSpan ? (uint32_t)left : kGeluSpan;
+  const rsrc_t ri = make_rsrc(reinterpret_cast<const char*>(in) + span0, span_bytes);
+  const rsrc_t ro = make_rsrc(reinterpret_cast<char*>(out) + span0, span_bytes);
+  const uint32_t off = (blockIdx.x * kRowSeg + threadIdx.x) * 16u;
+  Vec<DT> x;
+  x.unpack(buf_load16<kStreamLoad>(ri, off));
 #pragma unroll
-  for (int u = 0; u < UNROLL; ++u) {
-    int64_t v = base + (int64_t)u * kActBlock;
-    if (v < n16) raw[u] = load16_stream(in, v);
-  }
-#pragma unroll
-  for (int u = 0; u < UNROLL; ++u) {
-    int64_t v = base + (int64_t)u * kActBlock;
-    if (v < n16) {
-      Vec<DT> x;
-      x.unpack(raw[u]);
-#pragma unroll
-      for (int i = 0; i < N; ++i)
-        x.f[i] = FAST ? gelu_fast_elem<DT>(x.f[i]) : gelu_new_elem<DT>(x.f[i]);
-      store16_stream(out, v, x.pack());
-    }
-  }
-  // tail elements (numel not a multiple of the vector width): first block only
-  if (blockIdx.x == 0) {
-    int64_t i = n16 * N + threadIdx.x;
+  for (int i = 0; i < N; ++i)
+    x.f[i] = FAST ? gelu_fast_elem<DT>(x.f[i]) : gelu_new_elem<DT>(x.f[i]);
+  buf_store16<kStreamStore>(ro, off, x.pack());
+  if (blockIdx.x == 0 && blockIdx.y == 0) {
+    const int64_t i = vec_bytes / ElemBytes<DT>::value + threadIdx.x;
     if (i < numel) {
-      float x = load_elem<DT>(in, i);
-      store_elem<DT>(out, i, FAST ? gelu_fast_elem<DT>(x) : gelu_new_elem<DT>(x));
+      float v = load_elem<DT>(in, i);
+      store_elem<DT>(out, i, FAST ? gelu_fast_elem<DT>(v) : gelu_new_elem<DT>(v));
     }
   }
 }
@@ -172,7 +174,6 @@ __global__ __launch_bounds__(kActBlock) void gelu_scalar_kernel(void* __restrict
 template <int DT, bool FAST>
 static int launch_gelu(void* out, const void* in, int64_t numel, hipStream_t st) {
   constexpr int N = VecElems<DT>::value;
-  constexpr int UNROLL = 4;
   if (!(aligned16(out) && aligned16(in))) {
     int64_t blocks = (numel + kActBlock - 1) / kActBlock;
     if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
@@ -180,12 +181,15 @@ static int launch_gelu(void* out, const void* in, int64_t numel, hipStream_t st)
                        st, out, in, numel);
     return launch_status();
   }
-  const int64_t n16 = numel / N;
-  int64_t blocks = (n16 + (int64_t)UNROLL * kActBlock - 1) / ((int64_t)UNROLL * kActBlock);
-  if (blocks < 1) blocks = 1;
-  if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL((gelu_kernel<DT, FAST, UNROLL>), dim3((unsigned)blocks), dim3(kActBlock), 0,
-                     st, out, in, n16, numel);
+  const int64_t vec_bytes = numel / N * 16;
+  int64_t spans = (vec_bytes + kGeluSpan - 1) / kGeluSpan;
+  if (spans < 1) spans = 1;
+  if (spans > kMaxGridY) return SARATHI_ERR_UNSUPPORTED;
+  const int64_t first_span = vec_bytes < (int64_t)kGeluSpan ? vec_bytes : (int64_t)kGeluSpan;
+  int64_t segs = (first_span / 16 + kRowSeg - 1) / kRowSeg;
+  if (segs < 1) segs = 1;
+  hipLaunchKernelGGL((gelu_kernel<DT, FAST>), dim3((unsigned)segs, (unsigned)spans), dim3(kRowSeg),
+                     0, st, out, in, vec_bytes, numel);
   return launch_status();
 }
 

@@ -61,11 +61,11 @@ __global__ __launch_bounds__(kTopkBlock) void topk_softmax_pow2_kernel(
     if constexpr (L::ELTS == 4) {
       u32x4 q = *reinterpret_cast<const u32x4*>(p);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[l * 4 + i] = __builtin_bit_cast(float, q[i]);
+      for (int i = 0; i < 4; ++i) v[l * 4 + i] = as_f32(q[i]);
     } else if constexpr (L::ELTS == 2) {
       u32x2 q = *reinterpret_cast<const u32x2*>(p);
-      v[0] = __builtin_bit_cast(float, q.x);
-      v[1] = __builtin_bit_cast(float, q.y);
+      v[0] = as_f32(q.x);
+      v[1] = as_f32(q.y);
     } else {
       v[0] = p[0];
     }

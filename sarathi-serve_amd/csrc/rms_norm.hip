@@ -2,11 +2,14 @@
 //
 // Replaces csrc/layernorm_kernels.cu:11-62 of the reference (one 1024-thread
 // block per token, 2-byte loads, the row read twice, a two-level shared-memory
-// reduction).  Here one 64-lane wave owns one token row and keeps it in
+// reduction).  Here one small workgroup owns one token row and keeps it in
 // registers: the row is read from HBM exactly once with 16-byte loads that are
-// all issued before the first use, the sum of squares is folded inside the wave
-// with DPP, and the normalised row is written with 16-byte stores.  No LDS and
-// no barrier.  A block is four independent waves (four rows).
+// all issued before the first use, and written with 16-byte stores.  A lane
+// holds at most four vectors, so a row of H elements takes H/32 lanes (bf16):
+// 128 lanes at H = 4096, 256 at H = 8192.  Many small workgroups whose ids walk
+// memory linearly measured faster on MI355X than fewer, fatter ones.  The sum
+// of squares is folded inside each wave with DPP; waves of a row combine
+// through one LDS word each and a single barrier.
 //
 // Arithmetic (rounding points as in the reference):
 //   ss = sum f32(x)^2 ; s = rsqrt(ss / H + eps)
@@ -17,36 +20,31 @@
 
 namespace sarathi_hip {
 
-constexpr int kRmsWavesPerBlock = 4;
-
-// VPL = 16-byte vectors held per lane; the row has nvec <= 64 * VPL vectors.
-template <int DT, int VPL, bool FUSED>
-__global__ __launch_bounds__(64 * kRmsWavesPerBlock) void rms_norm_wave_kernel(
+// WAVES = waves per row (1, 2, 4, 8 or 16), VPL = 16-byte vectors per lane;
+// the row has nvec <= 64 * WAVES * VPL vectors.
+template <int DT, int WAVES, int VPL, bool FUSED>
+__global__ __launch_bounds__(64 * WAVES) void rms_norm_row_kernel(
     void* out,        // FUSED: the `input` tensor, updated in place
     void* in_or_res,  // FUSED: the residual tensor, updated in place
-    const void* __restrict__ weight, float eps, int64_t num_tokens, int nvec, float hidden_f,
-    int64_t out_stride_vec, int64_t in_stride_vec) {
+    const void* __restrict__ weight, float eps, uint32_t row_bytes, float hidden_f,
+    int64_t out_stride_bytes, int64_t in_stride_bytes) {
   constexpr int N = VecElems<DT>::value;
-  const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * kRmsWavesPerBlock + (threadIdx.x >> 6);
-  if (row >= num_tokens) return;  // wave-uniform
+  constexpr int TPR = 64 * WAVES;
+  __shared__ float partial[WAVES];
+  const int64_t row = blockIdx.x;
+  const rsrc_t rin = make_rsrc(reinterpret_cast<char*>(in_or_res) + row * in_stride_bytes, row_bytes);
+  const rsrc_t rout = make_rsrc(reinterpret_cast<char*>(out) + row * out_stride_bytes, row_bytes);
+  const rsrc_t rw = make_rsrc(weight, row_bytes);
+  const uint32_t off0 = threadIdx.x * 16u;
 
-  const int64_t in_base = row * in_stride_vec;
-  const int64_t out_base = row * out_stride_vec;
-
+  // lanes past the end of the row read zeros and their stores are dropped
   u32x4 raw[VPL];
 #pragma unroll
-  for (int j = 0; j < VPL; ++j) {
-    int c = lane + 64 * j;
-    raw[j] = c < nvec ? load16_stream(in_or_res, in_base + c) : (u32x4){0, 0, 0, 0};
-  }
+  for (int j = 0; j < VPL; ++j) raw[j] = buf_load16<kStreamLoad>(rin, off0 + j * (TPR * 16u));
   if constexpr (FUSED) {
     u32x4 hid[VPL];
 #pragma unroll
-    for (int j = 0; j < VPL; ++j) {
-      int c = lane + 64 * j;
-      hid[j] = c < nvec ? load16_stream(out, out_base + c) : (u32x4){0, 0, 0, 0};
-    }
+    for (int j = 0; j < VPL; ++j) hid[j] = buf_load16<kStreamLoad>(rout, off0 + j * (TPR * 16u));
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
       Vec<DT> a, b;
@@ -55,19 +53,14 @@ __global__ __launch_bounds__(64 * kRmsWavesPerBlock) void rms_norm_wave_kernel(
 #pragma unroll
       for (int i = 0; i < N; ++i) a.f[i] = b.f[i] + a.f[i];
       raw[j] = a.pack();  // z, rounded to the dtype
-      int c = lane + 64 * j;
-      if (c < nvec) store16_stream(in_or_res, in_base + c, raw[j]);
+      buf_store16<kStreamStore>(rin, off0 + j * (TPR * 16u), raw[j]);
     }
   }
-
   // weight vectors are shared by every row and stay cache resident; fetch them
   // now so their latency overlaps the reduction
   u32x4 wraw[VPL];
 #pragma unroll
-  for (int j = 0; j < VPL; ++j) {
-    int c = lane + 64 * j;
-    wraw[j] = c < nvec ? load16(weight, c) : (u32x4){0, 0, 0, 0};
-  }
+  for (int j = 0; j < VPL; ++j) wraw[j] = buf_load16<kCached>(rw, off0 + j * (TPR * 16u));
 
   float ss = 0.f;
 #pragma unroll
@@ -78,19 +71,24 @@ __global__ __launch_bounds__(64 * kRmsWavesPerBlock) void rms_norm_wave_kernel(
     for (int i = 0; i < N; ++i) ss = __builtin_fmaf(a.f[i], a.f[i], ss);
   }
   ss = wave64_sum(ss);
+  if constexpr (WAVES > 1) {
+    if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    float t = partial[0];
+#pragma unroll
+    for (int k = 1; k < WAVES; ++k) t += partial[k];
+    ss = t;
+  }
   const float s = __builtin_amdgcn_rsqf(ss / hidden_f + eps);
 
 #pragma unroll
   for (int j = 0; j < VPL; ++j) {
-    int c = lane + 64 * j;
-    if (c < nvec) {
-      Vec<DT> a, w;
-      a.unpack(raw[j]);
-      w.unpack(wraw[j]);
+    Vec<DT> a, w;
+    a.unpack(raw[j]);
+    w.unpack(wraw[j]);
 #pragma unroll
-      for (int i = 0; i < N; ++i) a.f[i] = rnd<DT>(a.f[i] * s) * w.f[i];
-      store16_stream(out, out_base + c, a.pack());
-    }
+    for (int i = 0; i < N; ++i) a.f[i] = rnd<DT>(a.f[i] * s) * w.f[i];
+    buf_store16<kStreamStore>(rout, off0 + j * (TPR * 16u), a.pack());
   }
 }
 
@@ -127,28 +125,30 @@ template <int DT, bool FUSED>
 static int launch_rms(void* out, void* in, const void* w, float eps, int64_t T, int64_t H,
                       int64_t out_stride, int64_t in_stride, hipStream_t st) {
   constexpr int N = VecElems<DT>::value;
+  constexpr int EB = ElemBytes<DT>::value;
   const float hidden_f = (float)H;
+  if (T > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
   const bool vec_ok = (H % N == 0) && (out_stride % N == 0) && (in_stride % N == 0) &&
-                      aligned16(out) && aligned16(in) && aligned16(w) && (H / N) <= 64 * 16;
+                      aligned16(out) && aligned16(in) && aligned16(w) && (H / N) <= 1024 * 4;
   if (!vec_ok) {
-    if (T > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((rms_norm_generic_kernel<DT, FUSED>), dim3((unsigned)T), dim3(256), 0, st,
                        out, in, w, eps, (int)H, hidden_f, out_stride, in_stride);
     return launch_status();
   }
   const int nvec = (int)(H / N);
-  const int64_t blocks = (T + kRmsWavesPerBlock - 1) / kRmsWavesPerBlock;
-  if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
-  dim3 grid((unsigned)blocks), block(64 * kRmsWavesPerBlock);
-  const int vpl = (nvec + 63) / 64;
-#define SK_RMS_CASE(V)                                                                        \
-  hipLaunchKernelGGL((rms_norm_wave_kernel<DT, V, FUSED>), grid, block, 0, st, out, in, w, eps, \
-                     T, nvec, hidden_f, out_stride / N, in_stride / N)
-  if (vpl <= 1) SK_RMS_CASE(1);
-  else if (vpl <= 2) SK_RMS_CASE(2);
-  else if (vpl <= 4) SK_RMS_CASE(4);
-  else if (vpl <= 8) SK_RMS_CASE(8);
-  else SK_RMS_CASE(16);
+  const uint32_t row_bytes = (uint32_t)(H * EB);
+  dim3 grid((unsigned)T);
+#define SK_RMS_CASE(WAVES, VPL)                                                               \
+  hipLaunchKernelGGL((rms_norm_row_kernel<DT, WAVES, VPL, FUSED>), grid, dim3(64 * WAVES), 0, \
+                     st, out, in, w, eps, row_bytes, hidden_f, out_stride * EB, in_stride * EB)
+  // four vectors per lane once the row is long enough, never more than 1024 lanes
+  if (nvec <= 64) SK_RMS_CASE(1, 1);
+  else if (nvec <= 128) SK_RMS_CASE(1, 2);
+  else if (nvec <= 256) SK_RMS_CASE(1, 4);
+  else if (nvec <= 512) SK_RMS_CASE(2, 4);
+  else if (nvec <= 1024) SK_RMS_CASE(4, 4);
+  else if (nvec <= 2048) SK_RMS_CASE(8, 4);
+  else SK_RMS_CASE(16, 4);
 #undef SK_RMS_CASE
   return launch_status();
 }

@@ -9,11 +9,13 @@
 //          them in registers and writes both vectors back;
 //   GPT-J: x and y interleave, so one 16-byte vector already holds whole
 //          pairs; cos and sin come from two half-width loads.
-// threadIdx.x walks the slots of a head and threadIdx.y the heads (q heads
-// first, then k heads), so no integer division is needed, and each thread
-// handles TOK consecutive tokens with all loads issued first.  Row offsets are
-// 64-bit.  q and k rows may be views into a packed qkv buffer (row stride !=
-// row width); elements at or beyond rot_dim inside a head are not touched.
+// A workgroup is one wave: 64 consecutive slots of one token's q row or of its
+// k row (8 heads of 128 at bf16).  Workgroup ids run over the q segments, then
+// the k segments, then the tokens, so the waves in flight sweep the packed qkv
+// buffer linearly.  The token's q row, k row and cos/sin cache row are scalar
+// buffer resources (the position is a scalar load); lanes past the last head
+// are clipped by the hardware range check, so the kernel has no branches.
+// Elements at or beyond rot_dim inside a head are not touched.
 //
 // Arithmetic is the reference's scalar_t arithmetic: each product and the final
 // sum round to the tensor dtype (csrc/pos_encoding_kernels.cu:32-35):
@@ -22,6 +24,9 @@
 #include "launch.h"
 
 namespace sarathi_hip {
+
+constexpr int kMaxGridY = 65535;
+constexpr uint32_t kClipped = 0x80000000u;  // byte offset beyond any row: access is dropped
 
 struct RopeArgs {
   const int64_t* positions;
@@ -39,74 +44,60 @@ struct RopeArgs {
 
 template <int DT> SK_DEV float mul_r(float a, float b) { return rnd<DT>(a * b); }
 
-template <int DT, bool NEOX, int TOK>
-__global__ __launch_bounds__(1024) void rope_vec_kernel(RopeArgs a) {
+// slots = 16-byte slots per head (NeoX: of the x half; GPT-J: of the rotated span);
+// slot_shift = log2(slots) or -1 when slots is not a power of two.
+template <int DT, bool NEOX>
+__global__ __launch_bounds__(64) void rope_seg_kernel(RopeArgs a, int64_t tok0, int q_blocks,
+                                                      int slots, int slot_shift) {
   constexpr int N = VecElems<DT>::value;
-  const int slot = threadIdx.x;  // 16-byte slot inside the head's x half (NeoX) / head (GPT-J)
-  const int total_heads = a.num_heads + a.num_kv_heads;
-  const int64_t tok0 = (int64_t)blockIdx.x * TOK;
-  const int embed = a.rot_dim >> 1;
+  constexpr int EB = ElemBytes<DT>::value;
+  const int64_t tok = tok0 + (int64_t)blockIdx.z * kMaxGridY + blockIdx.y;
+  const bool is_q = (int)blockIdx.x < q_blocks;  // uniform over the wave
+  const int item = ((int)blockIdx.x - (is_q ? 0 : q_blocks)) * 64 + (int)threadIdx.x;
+  const int nheads = is_q ? a.num_heads : a.num_kv_heads;
+  int h, slot;
+  if (slot_shift >= 0) {
+    h = item >> slot_shift;
+    slot = item & (slots - 1);
+  } else {
+    h = item / slots;
+    slot = item - h * slots;
+  }
+  const uint32_t embed_bytes = (uint32_t)(a.rot_dim >> 1) * EB;
+  char* base = reinterpret_cast<char*>(is_q ? a.query : a.key) +
+               tok * (is_q ? a.q_stride : a.k_stride) * EB;
+  const rsrc_t rd = make_rsrc(base, (uint32_t)nheads * a.head_size * EB);
+  const rsrc_t rc = make_rsrc(
+      reinterpret_cast<const char*>(a.cache) + a.positions[tok] * a.rot_dim * EB, 2 * embed_bytes);
+  const uint32_t xoff = h < nheads ? (uint32_t)h * a.head_size * EB + slot * 16u : kClipped;
 
-  for (int head = threadIdx.y; head < total_heads; head += blockDim.y) {
-    const bool is_q = head < a.num_heads;
-    char* base = reinterpret_cast<char*>(is_q ? a.query : a.key);
-    const int64_t stride = is_q ? a.q_stride : a.k_stride;
-    const int h = is_q ? head : head - a.num_heads;
-    constexpr int EB = ElemBytes<DT>::value;
-
-    u32x4 xv[TOK], yv[TOK], cv[TOK], sv[TOK];
-    char* xp[TOK];
+  if constexpr (NEOX) {
+    Vec<DT> x, y, c, s, ox, oy;
+    x.unpack(buf_load16<kStreamLoad>(rd, xoff));
+    y.unpack(buf_load16<kStreamLoad>(rd, xoff + embed_bytes));
+    c.unpack(buf_load16<kCached>(rc, slot * 16u));
+    s.unpack(buf_load16<kCached>(rc, embed_bytes + slot * 16u));
 #pragma unroll
-    for (int t = 0; t < TOK; ++t) {
-      const int64_t tok = tok0 + t;
-      if (tok < a.num_tokens) {
-        xp[t] = base + (tok * stride + (int64_t)h * a.head_size) * EB;
-        const char* crow =
-            reinterpret_cast<const char*>(a.cache) + a.positions[tok] * a.rot_dim * EB;
-        if constexpr (NEOX) {
-          xv[t] = *reinterpret_cast<const u32x4*>(xp[t] + slot * 16);
-          yv[t] = *reinterpret_cast<const u32x4*>(xp[t] + embed * EB + slot * 16);
-          cv[t] = *reinterpret_cast<const u32x4*>(crow + slot * 16);
-          sv[t] = *reinterpret_cast<const u32x4*>(crow + embed * EB + slot * 16);
-        } else {
-          xv[t] = *reinterpret_cast<const u32x4*>(xp[t] + slot * 16);
-          u32x2 c2 = *reinterpret_cast<const u32x2*>(crow + slot * 8);
-          u32x2 s2 = *reinterpret_cast<const u32x2*>(crow + embed * EB + slot * 8);
-          cv[t] = (u32x4){c2.x, c2.y, 0, 0};
-          sv[t] = (u32x4){s2.x, s2.y, 0, 0};
-        }
-      }
+    for (int i = 0; i < N; ++i) {
+      ox.f[i] = mul_r<DT>(x.f[i], c.f[i]) - mul_r<DT>(y.f[i], s.f[i]);
+      oy.f[i] = mul_r<DT>(y.f[i], c.f[i]) + mul_r<DT>(x.f[i], s.f[i]);
     }
+    buf_store16<kStreamStore>(rd, xoff, ox.pack());
+    buf_store16<kStreamStore>(rd, xoff + embed_bytes, oy.pack());
+  } else {
+    Vec<DT> x, c, s, o;
+    x.unpack(buf_load16<kStreamLoad>(rd, xoff));
+    const u32x2 c2 = buf_load8<kCached>(rc, slot * 8u);
+    const u32x2 s2 = buf_load8<kCached>(rc, embed_bytes + slot * 8u);
+    c.unpack((u32x4){c2.x, c2.y, 0, 0});
+    s.unpack((u32x4){s2.x, s2.y, 0, 0});
 #pragma unroll
-    for (int t = 0; t < TOK; ++t) {
-      const int64_t tok = tok0 + t;
-      if (tok < a.num_tokens) {
-        Vec<DT> x, y, c, s;
-        x.unpack(xv[t]);
-        c.unpack(cv[t]);
-        s.unpack(sv[t]);
-        if constexpr (NEOX) {
-          y.unpack(yv[t]);
-          Vec<DT> ox, oy;
-#pragma unroll
-          for (int i = 0; i < N; ++i) {
-            ox.f[i] = mul_r<DT>(x.f[i], c.f[i]) - mul_r<DT>(y.f[i], s.f[i]);
-            oy.f[i] = mul_r<DT>(y.f[i], c.f[i]) + mul_r<DT>(x.f[i], s.f[i]);
-          }
-          *reinterpret_cast<u32x4*>(xp[t] + slot * 16) = ox.pack();
-          *reinterpret_cast<u32x4*>(xp[t] + embed * EB + slot * 16) = oy.pack();
-        } else {
-          Vec<DT> o;
-#pragma unroll
-          for (int i = 0; i < N / 2; ++i) {
-            float xe = x.f[2 * i], ye = x.f[2 * i + 1];
-            o.f[2 * i] = mul_r<DT>(xe, c.f[i]) - mul_r<DT>(ye, s.f[i]);
-            o.f[2 * i + 1] = mul_r<DT>(ye, c.f[i]) + mul_r<DT>(xe, s.f[i]);
-          }
-          *reinterpret_cast<u32x4*>(xp[t] + slot * 16) = o.pack();
-        }
-      }
+    for (int i = 0; i < N / 2; ++i) {
+      const float xe = x.f[2 * i], ye = x.f[2 * i + 1];
+      o.f[2 * i] = mul_r<DT>(xe, c.f[i]) - mul_r<DT>(ye, s.f[i]);
+      o.f[2 * i + 1] = mul_r<DT>(ye, c.f[i]) + mul_r<DT>(xe, s.f[i]);
     }
+    buf_store16<kStreamStore>(rd, xoff, o.pack());
   }
 }
 
@@ -141,23 +132,35 @@ static int launch_rope(const RopeArgs& a, hipStream_t st) {
   // 16-byte slots per head: NeoX covers the x half (the y half rides along), GPT-J the whole
   // rotated span
   const int span = NEOX ? embed : a.rot_dim;
-  const bool vec_ok = (span % N == 0) && (span / N <= 1024) && ((a.head_size * EB) % 16 == 0) &&
+  const int64_t q_row_bytes = (int64_t)a.num_heads * a.head_size * EB;
+  const int64_t k_row_bytes = (int64_t)a.num_kv_heads * a.head_size * EB;
+  const bool vec_ok = (span % N == 0) && ((a.head_size * EB) % 16 == 0) &&
                       ((a.q_stride * EB) % 16 == 0) && ((a.k_stride * EB) % 16 == 0) &&
                       ((a.rot_dim * EB) % 16 == 0) && ((embed * EB) % (NEOX ? 16 : 8) == 0) &&
-                      aligned16(a.query) && aligned16(a.key) && aligned16(a.cache);
+                      aligned16(a.query) && aligned16(a.key) && aligned16(a.cache) &&
+                      q_row_bytes < (int64_t)kClipped && k_row_bytes < (int64_t)kClipped;
   if (!vec_ok) {
     hipLaunchKernelGGL((rope_generic_kernel<DT, NEOX>), dim3((unsigned)a.num_tokens), dim3(256),
                        0, st, a);
     return launch_status();
   }
-  constexpr int TOK = 2;
   const int slots = span / N;
-  const int heads = a.num_heads + a.num_kv_heads;
-  int by = 1024 / slots;
-  if (by > heads) by = heads;
-  dim3 block((unsigned)slots, (unsigned)by);
-  dim3 grid((unsigned)((a.num_tokens + TOK - 1) / TOK));
-  hipLaunchKernelGGL((rope_vec_kernel<DT, NEOX, TOK>), grid, block, 0, st, a);
+  int slot_shift = -1;
+  if ((slots & (slots - 1)) == 0) {
+    slot_shift = 0;
+    while ((1 << slot_shift) < slots) ++slot_shift;
+  }
+  const int64_t q_blocks = ((int64_t)a.num_heads * slots + 63) / 64;
+  const int64_t k_blocks = ((int64_t)a.num_kv_heads * slots + 63) / 64;
+  if (q_blocks + k_blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
+  const unsigned gx = (unsigned)(q_blocks + k_blocks);
+  const int64_t full_z = a.num_tokens / kMaxGridY, rem = a.num_tokens % kMaxGridY;
+  if (full_z > 0)
+    hipLaunchKernelGGL((rope_seg_kernel<DT, NEOX>), dim3(gx, kMaxGridY, (unsigned)full_z), dim3(64),
+                       0, st, a, (int64_t)0, (int)q_blocks, slots, slot_shift);
+  if (rem > 0)
+    hipLaunchKernelGGL((rope_seg_kernel<DT, NEOX>), dim3(gx, (unsigned)rem, 1), dim3(64), 0, st, a,
+                       full_z * kMaxGridY, (int)q_blocks, slots, slot_shift);
   return launch_status();
 }
 

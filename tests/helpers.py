@@ -34,28 +34,39 @@ def cos_sin_cache(max_pos, rot_dim, theta, dtype):
 
 
 def ulp_of(t):
-    """Spacing of the tensor's dtype at each element's magnitude (as float32)."""
+    """Spacing of the tensor's dtype at each element's magnitude (as float32).  Magnitudes below
+    2^-100 are treated as 2^-100: differences down there are flush-to-zero effects of the hardware
+    reciprocal, far below anything the stated tolerance can see."""
     mant = {torch.bfloat16: 7, torch.float16: 10, torch.float32: 23}[t.dtype]
-    mag = t.float().abs().clamp_min(2.0 ** -126)
+    mag = t.float().abs().clamp_min(2.0 ** -100)
     return torch.exp2(torch.floor(torch.log2(mag)) - mant)
 
 
-def assert_close_dtype(got, want, atol=1e-2, rtol=1e-2, max_ulps=1, max_mismatch_frac=5e-3):
+def assert_close_dtype(got, want, atol=1e-2, rtol=1e-2, max_ulps=2, max_mismatch_frac=5e-3):
     """The stated tolerance (|got-want| <= atol + rtol*|want|, i.e. torch.allclose semantics with
     atol = rtol = 1e-2) plus the much tighter bound the kernels actually meet: no element is off
     by more than `max_ulps` units in the last place of the dtype and only a small fraction is off
-    at all."""
+    at all.  Ops that round twice (rms_norm, silu_and_mul) can turn a one-ulp flip of the
+    intermediate into two ulps of the result, hence the default of 2.  Non-finite values must
+    match exactly.  max_ulps=None skips the ulp bound (fp32 outputs, where reduction order and
+    the transcendental's last place show directly)."""
     got, want = got.cpu(), want.cpu()
     assert got.shape == want.shape and got.dtype == want.dtype
     g, w = got.float(), want.float()
-    assert torch.isfinite(g).all() == torch.isfinite(w).all()
+    fin = torch.isfinite(w)
+    assert torch.equal(torch.isfinite(g), fin), "non-finite positions differ"
+    assert torch.equal(g[~fin].nan_to_num(nan=7.0), w[~fin].nan_to_num(nan=7.0))
+    g, w = g[fin], w[fin]
     diff = (g - w).abs()
+    if diff.numel() == 0:
+        return 0.0
     assert bool((diff <= atol + rtol * w.abs()).all()), (
         "outside tolerance: max abs %.4g" % diff.max().item())
     bad = diff > 0
     frac = bad.float().mean().item()
-    if bad.any():
-        ulps = (diff / torch.maximum(ulp_of(got), ulp_of(want)))[bad].max().item()
+    if bad.any() and max_ulps is not None:
+        ulp = torch.maximum(ulp_of(got), ulp_of(want))[fin]
+        ulps = (diff / ulp)[bad].max().item()
         assert ulps <= max_ulps + 1e-3, "max error %.2f ulp" % ulps
     assert frac <= max_mismatch_frac, "mismatching fraction %.3g" % frac
     return frac

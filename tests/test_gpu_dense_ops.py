@@ -18,9 +18,11 @@ DTYPES = [torch.bfloat16, torch.float16, torch.float32]
 
 
 def _tol(dtype):
-    # fp32 results differ from the oracle only through exp / rsqrt / reduction order
-    return dict(atol=1e-2, rtol=1e-2, max_ulps=1 if dtype != torch.float32 else 64,
-                max_mismatch_frac=5e-3 if dtype != torch.float32 else 1.0)
+    if dtype == torch.float32:
+        # fp32 outputs show the reduction order and the last place of exp / rsqrt / tanh directly;
+        # bound them far inside the stated 1e-2 instead of counting ulps
+        return dict(atol=2e-6, rtol=2e-5, max_ulps=None, max_mismatch_frac=1.0)
+    return dict(atol=1e-2, rtol=1e-2, max_ulps=2, max_mismatch_frac=5e-3)
 
 
 # ---------------------------------------------------------------- rms_norm
@@ -158,7 +160,6 @@ def test_gelu_matches_oracle(ops, dev, dtype, name, T, d):
     getattr(ops.activation_ops, name)(got, x.to(dev))
     # the chains of dtype roundings amplify a last-place difference in tanh by up to 2 ulp
     tol = _tol(dtype)
-    tol["max_ulps"] = max(tol["max_ulps"], 2)
     tol["max_mismatch_frac"] = max(tol["max_mismatch_frac"], 2e-2)
     assert_close_dtype(got, want, **tol)
 
