@@ -13,9 +13,14 @@ several independent buffer sets whose total footprint exceeds 512 MB, so the 256
 cannot serve the reads ("cold" numbers).  `value` is the step's algorithmic bytes divided by the
 step time.  `per_op` carries, for every op (plus rms_norm alone and the Mixtral-shaped MoE routing
 ops), µs per call, GB/s and fraction of the 8 TB/s HBM peak, cold and warm (same buffers every
-call).  `roofline` describes the dominant kernel of the step, silu_and_mul, timed with HIP events
-placed around that launch inside the timed region.  `cpu_baseline` is the PyTorch CPU formulation
-of the same step on this machine's host cores.
+call).  `roofline` describes the dominant kernel of the step, silu_and_mul: its algorithmic bytes
+divided by its average launch duration over --steps back-to-back launches on cold buffers between
+two HIP events on the launch stream.  `cpu_baseline` is the PyTorch CPU formulation of the same
+step on this machine's host cores.
+
+--calibrate-copy additionally runs a plain device-to-device copy of a known size (256 MiB,
+torch's copy kernel) so that a `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` run of this script can
+scale the counters by what they read for a known amount of traffic.
 
 Prints ONE JSON line.
 """
@@ -41,7 +46,8 @@ BF16 = 2
 BYTES = {
     "fused_add_rms_norm": 4 * T * H * BF16 + H * BF16,
     "rms_norm": 2 * T * H * BF16 + H * BF16,
-    "rotary_embedding": 2 * (T * NQ * D + T * NKV * D) * BF16 + T * 8,   # + touched cache rows
+    # q and k read + written, int64 positions, one cos||sin cache row per token
+    "rotary_embedding": 2 * (T * NQ * D + T * NKV * D) * BF16 + T * 8 + T * D * BF16,
     "silu_and_mul": (2 * T * DFF + T * DFF) * BF16,
 }
 MOE_T, MOE_E, MOE_K, MOE_B = 4096, 8, 2, 64
@@ -76,6 +82,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--sets", type=int, default=4, help="independent buffer sets to rotate through")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch a 256 MiB plain copy (counter calibration for --pmc runs)")
+    ap.add_argument("--traffic", type=float, default=None,
+                    help="measured HBM bytes per silu_and_mul launch (from a --pmc run), reported "
+                         "verbatim as roofline.traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this op library runs on one GPU; --gpus must be 1 "
@@ -96,15 +107,11 @@ def main():
     sets = [make_set(torch, g, dev, cache_cpu) for _ in range(args.sets)]
     set_bytes = sum(v.numel() * v.element_size() for k, v in sets[0].items() if k not in ("q", "k"))
 
-    def step(s, ev=None):
+    def step(s):
         LN.fused_add_rms_norm(s["x"], s["res"], s["w1"], 1e-5)
         ROPE.rotary_embedding(s["pos"], s["q"], s["k"], D, s["cache"], True)
         LN.fused_add_rms_norm(s["x"], s["res"], s["w2"], 1e-5)
-        if ev is not None:
-            ev[0].record()
         ACT.silu_and_mul(s["act"], s["gate_up"])
-        if ev is not None:
-            ev[1].record()
 
     step_bytes = 2 * BYTES["fused_add_rms_norm"] + BYTES["rotary_embedding"] + BYTES["silu_and_mul"]
 
@@ -112,20 +119,17 @@ def main():
     for i in range(args.warmup):
         step(sets[i % len(sets)])
     torch.cuda.synchronize()
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-           for _ in range(args.steps)]
     t0 = torch.cuda.Event(enable_timing=True)
     t1 = torch.cuda.Event(enable_timing=True)
     wall0 = time.perf_counter()
     t0.record()
     for i in range(args.steps):
-        step(sets[i % len(sets)], evs[i])
+        step(sets[i % len(sets)])
     t1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - wall0
     gpu_ms = t0.elapsed_time(t1)
     ms_per_step = max(gpu_ms, wall * 1e3) / args.steps
-    silu_us = sum(a.elapsed_time(b) for a, b in evs) * 1e3 / args.steps
 
     # ---- per-op tables: K back-to-back launches between two events ----
     # Every op gets its own ring of argument sets.  "cold": the ring's footprint exceeds
@@ -201,7 +205,7 @@ def main():
             if latency_bound and label == "cold":
                 continue   # 0.07-0.2 MB working sets: launch-latency-bound, one (warm) figure
             use = args_ring if label == "cold" else args_ring[:1]
-            us = time_op(fn, use, max(args.steps, 50))
+            us = time_op(fn, use, args.steps)
             gbs = BYTES[name] / us * 1e-3
             row[label] = {"us": round(us, 3), "GBps": round(gbs, 1),
                           "frac_of_peak": round(gbs / HBM_PEAK_GBS, 4)}
@@ -212,13 +216,23 @@ def main():
     del ops_table
     torch.cuda.empty_cache()
 
+    if args.calibrate_copy:
+        src = torch.empty((256 << 20) // 2, dtype=torch.bfloat16, device=dev).fill_(1.0)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
+    silu_us = per_op["silu_and_mul"]["cold"]["us"]
     silu_gbs = BYTES["silu_and_mul"] / silu_us * 1e-3
     roofline = {
         "kernel": "silu_and_mul_kernel (bf16, [2304, 28672] -> [2304, 14336])",
         "bound": "hbm", "achieved": round(silu_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": round(silu_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+        "frac": round(silu_gbs / HBM_PEAK_GBS, 4), "traffic": args.traffic,
         "bytes_per_launch": BYTES["silu_and_mul"], "avg_launch_us": round(silu_us, 3),
-        "timing": "hipEvent pair around each launch inside the timed region, cold buffers",
+        "timing": "%d back-to-back launches between two HIP events on the launch stream, rotating "
+                  "over %d cold buffer sets" % (args.steps, per_op["silu_and_mul"]["ring_sets"]),
     }
 
     # ---- CPU baseline: the PyTorch formulation of the same step on the host cores ----

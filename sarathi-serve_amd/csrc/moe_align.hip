@@ -7,15 +7,18 @@
 // (W = 16, or 8 above 512 experts) does the same sort with every lane busy:
 //
 //   1. count   wave w owns a contiguous, ascending chunk of the flat ids and
-//              reads it 64 ids at a time, coalesced.  Inside a 64-id tile the
-//              lanes that hold the same expert find each other with a
-//              bit-serial ballot match (log2(E) ballots), which gives every
-//              lane its rank among equal ids and the group's size; the first
-//              lane of each group adds the size to cnt[w][e] in LDS.
-//   2. scan    per expert, an exclusive scan of cnt[.][e] over the waves (LDS),
-//              then a wave-level prefix scan of the padded totals -> cumsum[].
-//   3. scatter every wave walks its chunk again: slot = cumsum[e] + cnt[w][e]
-//              + rank-in-tile, and the group leader bumps cnt[w][e].  Chunks
+//              reads it 64 ids at a time, coalesced (up to 8 tiles are loaded
+//              ahead, and a chunk of at most 8 tiles simply stays in registers
+//              for pass 3).  Inside a 64-id tile the lanes that hold the same
+//              expert find each other with a bit-serial ballot match (log2(E)
+//              ballots), which gives every lane its rank among equal ids and
+//              the group's size; the first lane of each group adds the size to
+//              cnt[e][w] in LDS.
+//   2. scan    per expert, an exclusive scan of cnt[e][.] over the waves done by
+//              W adjacent lanes with shuffles, then a wave-level prefix scan of
+//              the padded totals -> cumsum[].
+//   3. scatter every wave walks its chunk again: slot = cumsum[e] + cnt[e][w]
+//              + rank-in-tile, and the group leader bumps cnt[e][w].  Chunks
 //              are ascending and tiles are visited in order, so the order
 //              inside an expert is ascending token index, exactly the
 //              reference's (stable) order.
@@ -23,7 +26,8 @@
 //              set to numel, the caller-side `fill_` of
 //              sarathi/model_executor/layers/fused_moe/fused_moe.py:195.
 //
-// No atomics, no global scratch, bit-exact by construction.
+// Each LDS counter has a single writer wave, there is no global scratch and no
+// inter-workgroup traffic, so the result is deterministic and bit-exact.
 #include "vec16.h"
 #include "launch.h"
 
@@ -65,13 +69,13 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(
     const IdT* __restrict__ ids, int64_t numel, int E, int B, int nbits,
     int32_t* __restrict__ sorted, int64_t sorted_len, int32_t* __restrict__ expert_ids,
     int64_t expert_ids_len, int32_t* __restrict__ post_pad, int fill_pad) {
-  __shared__ int32_t cnt[kAlignCntInts];            // [W][E]
+  __shared__ int32_t cnt[kAlignCntInts];            // [E][W]: tokens of expert e in wave w's chunk
   __shared__ int32_t tot[kAlignMaxExperts];         // tokens per expert
   __shared__ int32_t cumsum[kAlignMaxExperts + 1];  // padded exclusive scan
 
   const int tid = threadIdx.x;
   const int nthr = blockDim.x;
-  const int W = nthr >> 6;
+  const int W = nthr >> 6;  // 16 or 8: a power of two
   const int wave = tid >> 6;
   const int lane = tid & 63;
 
@@ -84,38 +88,73 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(
   const int64_t tile_lo = wave * tiles_per_wave;
   int64_t tile_hi = tile_lo + tiles_per_wave;
   if (tile_hi > tiles_total) tile_hi = tiles_total;
-  int32_t* my_cnt = cnt + wave * E;
+  // small inputs: the wave's whole chunk stays in registers between the two passes
+  const bool resident = tiles_per_wave <= kAlignBatch;
 
-  // ---- 1. count
-  for (int64_t t0 = tile_lo; t0 < tile_hi; t0 += kAlignBatch) {
-    int e[kAlignBatch];
+  auto load_batch = [&](int64_t t0, int (&e)[kAlignBatch]) {
 #pragma unroll
     for (int u = 0; u < kAlignBatch; ++u) {
       const int64_t i = ((t0 + u) << 6) + lane;
       e[u] = (t0 + u < tile_hi && i < numel) ? checked_expert(ids[i], E) : -1;
     }
+  };
+  // cnt is indexed [e * W + wave]; only this wave touches its column, so plain LDS adds suffice
+  auto count_batch = [&](int64_t t0, const int (&e)[kAlignBatch]) {
 #pragma unroll
     for (int u = 0; u < kAlignBatch; ++u) {
       if (t0 + u < tile_hi) {  // wave-uniform
-        const bool valid = e[u] >= 0 && e[u] < E;
+        const bool valid = e[u] >= 0;
         const TileMatch m = match_expert(e[u], valid, nbits);
-        if (valid && m.rank == 0) my_cnt[e[u]] += m.count;
+        if (valid && m.rank == 0) atomicAdd(&cnt[e[u] * W + wave], m.count);
       }
+    }
+  };
+  auto scatter_batch = [&](int64_t t0, const int (&e)[kAlignBatch]) {
+#pragma unroll
+    for (int u = 0; u < kAlignBatch; ++u) {
+      if (t0 + u < tile_hi) {
+        const bool valid = e[u] >= 0;
+        const TileMatch m = match_expert(e[u], valid, nbits);
+        if (valid) {
+          int32_t* c = &cnt[e[u] * W + wave];
+          const int base = *c;  // every lane of the group reads before the leader's add below
+          const int64_t slot = (int64_t)cumsum[e[u]] + base + m.rank;
+          if (slot < sorted_len) sorted[slot] = (int32_t)(((t0 + u) << 6) + lane);
+          if (m.rank == 0) atomicAdd(c, m.count);
+        }
+      }
+    }
+  };
+
+  // ---- 1. count
+  int held[kAlignBatch];
+  if (resident) {
+    load_batch(tile_lo, held);
+    count_batch(tile_lo, held);
+  } else {
+    for (int64_t t0 = tile_lo; t0 < tile_hi; t0 += kAlignBatch) {
+      int e[kAlignBatch];
+      load_batch(t0, e);
+      count_batch(t0, e);
     }
   }
   __syncthreads();
 
-  // ---- 2. scan over waves per expert, then padded prefix over experts
-  for (int x = tid; x < E; x += nthr) {
-    int run = 0;
-    for (int w = 0; w < W; ++w) {
-      const int c = cnt[w * E + x];
-      cnt[w * E + x] = run;
-      run += c;
+  // ---- 2. exclusive scan over the W waves of every expert: W consecutive lanes own one expert
+  for (int i = tid; i < W * E; i += nthr) {
+    const int w = i & (W - 1);
+    const int c = cnt[i];
+    int x = c;
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+      const int y = __shfl_up(x, off, 16);
+      if (off < W && w >= off) x += y;
     }
-    tot[x] = run;
+    cnt[i] = x - c;
+    if (w == W - 1) tot[i / W] = x;
   }
   __syncthreads();
+  // padded prefix over the experts
   if (wave == 0) {
     int carry = 0;
     for (int base = 0; base < E; base += 64) {
@@ -137,51 +176,39 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(
   __syncthreads();
 
   // ---- 3. scatter
-  for (int64_t t0 = tile_lo; t0 < tile_hi; t0 += kAlignBatch) {
-    int e[kAlignBatch];
-#pragma unroll
-    for (int u = 0; u < kAlignBatch; ++u) {
-      const int64_t i = ((t0 + u) << 6) + lane;
-      e[u] = (t0 + u < tile_hi && i < numel) ? checked_expert(ids[i], E) : -1;
-    }
-#pragma unroll
-    for (int u = 0; u < kAlignBatch; ++u) {
-      if (t0 + u < tile_hi) {
-        const bool valid = e[u] >= 0 && e[u] < E;
-        const TileMatch m = match_expert(e[u], valid, nbits);
-        if (valid) {
-          const int base = my_cnt[e[u]];
-          const int64_t slot = (int64_t)cumsum[e[u]] + base + m.rank;
-          if (slot < sorted_len) sorted[slot] = (int32_t)(((t0 + u) << 6) + lane);
-          if (m.rank == 0) my_cnt[e[u]] = base + m.count;
-        }
-      }
+  if (resident) {
+    scatter_batch(tile_lo, held);
+  } else {
+    for (int64_t t0 = tile_lo; t0 < tile_hi; t0 += kAlignBatch) {
+      int e[kAlignBatch];
+      load_batch(t0, e);
+      scatter_batch(t0, e);
     }
   }
 
   // ---- 4. expert id of every block, padding slots
   const int total = cumsum[E];
   const int nblk = total / B;
-  auto expert_of = [&](int pos) {  // largest e with cumsum[e] <= pos, for pos < total
-    int lo = 0, hi = E;            // invariant: cumsum[lo] <= pos < cumsum[hi]
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (cumsum[mid] <= pos) lo = mid; else hi = mid;
+  for (int b = tid; b < nblk; b += nthr) {
+    if (b < expert_ids_len) {
+      const int pos = b * B;
+      int lo = 0, hi = E;  // invariant: cumsum[lo] <= pos < cumsum[hi]
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (cumsum[mid] <= pos) lo = mid; else hi = mid;
+      }
+      expert_ids[b] = lo;
     }
-    return lo;
-  };
-  for (int b = tid; b < nblk; b += nthr)
-    if (b < expert_ids_len) expert_ids[b] = expert_of(b * B);
+  }
   if (fill_pad) {
     const int32_t pad = (int32_t)numel;
-    for (int64_t i = tid; i < sorted_len; i += nthr) {
-      bool is_pad = true;
-      if (i < total) {
-        const int x = expert_of((int)i);
-        is_pad = (int)i - cumsum[x] >= tot[x];
-      }
-      if (is_pad) sorted[i] = pad;
+    // an expert's run ends with fewer than B padding slots
+    for (int64_t i = tid; i < (int64_t)E * B; i += nthr) {
+      const int x = (int)(i / B), j = (int)(i - (int64_t)x * B);
+      const int64_t slot = (int64_t)cumsum[x] + tot[x] + j;
+      if (slot < cumsum[x + 1]) sorted[slot] = pad;
     }
+    for (int64_t i = (int64_t)total + tid; i < sorted_len; i += nthr) sorted[i] = pad;
   }
 }
 

@@ -1,0 +1,129 @@
+"""The C-ABI shared library loads and exports every entry point that include/sarathi_ops.h
+declares; argument validation that happens before any GPU work returns the documented codes;
+the PyTorch front end refuses CPU tensors.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "sarathi_ops.h")
+LIB = os.path.join(ROOT, "sarathi-serve_amd", "sarathi_amd", "lib", "libsarathi_ops_hip.so")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sarathi_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    import sarathi_amd  # noqa: F401  loads torch (and with it the HIP runtime the library links to)
+    assert os.path.exists(LIB), "build the library first: python sarathi-serve_amd/build.py"
+    return ctypes.CDLL(LIB)
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_functions()
+    for n in ["sarathi_rms_norm", "sarathi_fused_add_rms_norm", "sarathi_silu_and_mul",
+              "sarathi_gelu_new", "sarathi_gelu_fast", "sarathi_rotary_embedding",
+              "sarathi_topk_softmax", "sarathi_moe_align_block_size", "sarathi_ops_abi_version",
+              "sarathi_ops_strerror"]:
+        assert n in names
+
+
+def test_library_exports_every_declared_symbol(lib):
+    for name in declared_functions():
+        assert hasattr(lib, name), "missing symbol " + name
+
+
+def test_version_and_error_strings(lib):
+    assert lib.sarathi_ops_abi_version() == 1
+    lib.sarathi_ops_strerror.restype = ctypes.c_char_p
+    assert lib.sarathi_ops_strerror(0) == b"ok"
+    for code in (-1, -2, -3, -99):
+        assert len(lib.sarathi_ops_strerror(code)) > 0
+
+
+def test_argument_validation_without_gpu(lib):
+    """Null pointers, negative sizes, bad strides and unknown dtype codes are rejected on the
+    host before anything is launched; zero tokens is a successful no-op."""
+    i64, f32, ci, vp = ctypes.c_int64, ctypes.c_float, ctypes.c_int, ctypes.c_void_p
+    buf = ctypes.create_string_buffer(256)
+    p = ctypes.cast(buf, vp)
+    null = vp(None)
+    INVALID, UNSUPPORTED, OK = -1, -2, 0
+    rms = lib.sarathi_rms_norm
+    assert rms(null, p, p, f32(1e-5), i64(1), i64(8), i64(8), i64(8), ci(2), null) == INVALID
+    assert rms(p, p, p, f32(1e-5), i64(-1), i64(8), i64(8), i64(8), ci(2), null) == INVALID
+    assert rms(p, p, p, f32(1e-5), i64(1), i64(8), i64(4), i64(8), ci(2), null) == INVALID  # stride < H
+    assert rms(p, p, p, f32(1e-5), i64(1), i64(8), i64(8), i64(8), ci(7), null) == UNSUPPORTED
+    assert rms(p, p, p, f32(1e-5), i64(0), i64(8), i64(8), i64(8), ci(2), null) == OK
+    fused = lib.sarathi_fused_add_rms_norm
+    assert fused(p, null, p, f32(1e-5), i64(1), i64(8), i64(8), i64(8), ci(2), null) == INVALID
+    assert fused(p, p, p, f32(1e-5), i64(0), i64(8), i64(8), i64(8), ci(2), null) == OK
+    silu = lib.sarathi_silu_and_mul
+    assert silu(p, null, i64(1), i64(8), i64(16), i64(8), ci(2), null) == INVALID
+    assert silu(p, p, i64(1), i64(8), i64(8), i64(8), ci(2), null) == INVALID      # stride < 2d
+    assert silu(p, p, i64(1), i64(8), i64(16), i64(8), ci(9), null) == UNSUPPORTED
+    assert silu(p, p, i64(0), i64(8), i64(16), i64(8), ci(2), null) == OK
+    for gelu in (lib.sarathi_gelu_new, lib.sarathi_gelu_fast):
+        assert gelu(null, p, i64(1), i64(8), ci(2), null) == INVALID
+        assert gelu(p, p, i64(1), i64(0), ci(2), null) == INVALID
+        assert gelu(p, p, i64(0), i64(8), ci(2), null) == OK
+    rope = lib.sarathi_rotary_embedding
+    args = lambda **kw: [kw.get("pos", p), p, p, kw.get("cache", p), i64(kw.get("T", 1)), ci(2), ci(1),  # noqa: E731
+                         ci(kw.get("hs", 16)), ci(kw.get("rot", 16)), i64(kw.get("qs", 32)), i64(16),
+                         ci(1), ci(kw.get("dt", 2)), null]
+    assert rope(*args(pos=null)) == INVALID
+    assert rope(*args(rot=15)) == INVALID            # odd rot_dim
+    assert rope(*args(rot=32)) == INVALID            # rot_dim > head_size
+    assert rope(*args(qs=16)) == INVALID             # stride < num_heads * head_size
+    assert rope(*args(dt=5)) == UNSUPPORTED
+    assert rope(*args(T=0)) == OK
+    topk = lib.sarathi_topk_softmax
+    assert topk(null, p, p, p, i64(1), ci(8), ci(2), ci(0), null) == INVALID
+    assert topk(p, p, p, p, i64(1), ci(8), ci(9), ci(0), null) == INVALID   # topk > experts
+    assert topk(p, p, p, p, i64(1), ci(0), ci(1), ci(0), null) == INVALID
+    assert topk(p, p, p, p, i64(1), ci(2048), ci(1), ci(0), null) == UNSUPPORTED
+    assert topk(p, p, p, p, i64(0), ci(8), ci(2), ci(0), null) == OK
+    align = lib.sarathi_moe_align_block_size
+    assert align(p, ci(3), i64(4), ci(8), ci(4), null, i64(64), p, i64(16), p, ci(0), null) == INVALID
+    assert align(p, ci(3), i64(4), ci(0), ci(4), p, i64(64), p, i64(16), p, ci(0), null) == INVALID
+    assert align(p, ci(3), i64(4), ci(8), ci(4), p, i64(8), p, i64(16), p, ci(0), null) == INVALID  # sorted too short
+    assert align(p, ci(3), i64(4), ci(8), ci(4), p, i64(64), p, i64(1), p, ci(0), null) == INVALID  # expert_ids too short
+    assert align(p, ci(3), i64(4), ci(4096), ci(4), p, i64(64), p, i64(16), p, ci(0), null) == UNSUPPORTED
+    assert align(p, ci(11), i64(4), ci(8), ci(4), p, i64(64), p, i64(16), p, ci(0), null) == UNSUPPORTED
+
+
+def test_front_end_refuses_cpu_tensors_and_bad_shapes(ops):
+    x = torch.zeros((2, 8), dtype=torch.bfloat16)
+    w = torch.ones(8, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="must live on the GPU"):
+        ops.layernorm_ops.rms_norm(torch.empty_like(x), x, w, 1e-5)
+    with pytest.raises(RuntimeError, match="must live on the GPU"):
+        ops.layernorm_ops.fused_add_rms_norm(x, x.clone(), w, 1e-5)
+    with pytest.raises(RuntimeError, match="must live on the GPU"):
+        ops.activation_ops.silu_and_mul(torch.empty((2, 4), dtype=torch.bfloat16), x)
+    with pytest.raises(RuntimeError, match="must live on the GPU"):
+        ops.pos_encoding_ops.rotary_embedding(torch.zeros(2, dtype=torch.int64), x, x.clone(), 8,
+                                              torch.zeros((4, 8), dtype=torch.bfloat16), True)
+    with pytest.raises(RuntimeError, match="must live on the GPU"):
+        ops.moe_ops.topk_softmax(torch.empty((2, 2)), torch.empty((2, 2), dtype=torch.int32),
+                                 torch.empty((2, 2), dtype=torch.int32), torch.zeros((2, 8)))
+    with pytest.raises(RuntimeError, match="must live on the GPU"):
+        ops.moe_ops.moe_align_block_size(torch.zeros((2, 2), dtype=torch.int32), 8, 4,
+                                         torch.empty(36, dtype=torch.int32),
+                                         torch.empty(9, dtype=torch.int32),
+                                         torch.empty(1, dtype=torch.int32))
+
+
+def test_op_namespaces_match_the_reference_module_surface(ops):
+    """Attribute names of the four pybind modules the reference builds (setup.py:95-136)."""
+    assert {"rms_norm", "fused_add_rms_norm"} <= set(dir(ops.layernorm_ops))
+    assert {"silu_and_mul", "gelu_new", "gelu_fast"} <= set(dir(ops.activation_ops))
+    assert {"rotary_embedding"} <= set(dir(ops.pos_encoding_ops))
+    assert {"topk_softmax", "moe_align_block_size"} <= set(dir(ops.moe_ops))
