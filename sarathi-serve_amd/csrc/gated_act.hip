@@ -24,7 +24,6 @@ namespace sarathi_hip {
 
 constexpr int kActBlock = 256;   // element-wise fallback kernels
 constexpr int kRowSeg = 64;      // lanes per workgroup of the streaming kernels
-constexpr int kMaxGridY = 65535;
 
 SK_DEV float silu_f32(float x) {
   // x * sigmoid(x) = x / (1 + 2^(-x * log2 e))

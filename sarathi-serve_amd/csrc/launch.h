@@ -9,6 +9,9 @@
 
 namespace sarathi_hip {
 
+// grid.y / grid.z limit of a launch; token rows above it spill into grid.z
+constexpr int kMaxGridY = 65535;
+
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // Status of the launch just issued on this thread (hipGetLastError is

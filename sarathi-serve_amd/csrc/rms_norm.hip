@@ -4,12 +4,11 @@
 // block per token, 2-byte loads, the row read twice, a two-level shared-memory
 // reduction).  Here one small workgroup owns one token row and keeps it in
 // registers: the row is read from HBM exactly once with 16-byte loads that are
-// all issued before the first use, and written with 16-byte stores.  A lane
-// holds at most four vectors, so a row of H elements takes H/32 lanes (bf16):
-// 128 lanes at H = 4096, 256 at H = 8192.  Many small workgroups whose ids walk
-// memory linearly measured faster on MI355X than fewer, fatter ones.  The sum
-// of squares is folded inside each wave with DPP; waves of a row combine
-// through one LDS word each and a single barrier.
+// all issued before the first use, and written with 16-byte stores.  Workgroup
+// ids walk the rows, i.e. memory, linearly.  How many lanes share a row is
+// chosen per shape (see launch_rms): a single wave per row where that fits,
+// otherwise 2..16 waves.  The sum of squares is folded inside each wave with
+// DPP; the waves of a row combine through one LDS word each and one barrier.
 //
 // Arithmetic (rounding points as in the reference):
 //   ss = sum f32(x)^2 ; s = rsqrt(ss / H + eps)
@@ -141,14 +140,25 @@ static int launch_rms(void* out, void* in, const void* w, float eps, int64_t T, 
 #define SK_RMS_CASE(WAVES, VPL)                                                               \
   hipLaunchKernelGGL((rms_norm_row_kernel<DT, WAVES, VPL, FUSED>), grid, dim3(64 * WAVES), 0, \
                      st, out, in, w, eps, row_bytes, hidden_f, out_stride * EB, in_stride * EB)
-  // four vectors per lane once the row is long enough, never more than 1024 lanes
+  // Shapes measured on MI355X at H = 4096 and H = 8192 (bf16).  The plain norm is fastest
+  // with a whole row of up to 512 vectors in ONE wave (no LDS, no barrier) and four vectors
+  // per lane beyond that; the fused op, which holds two rows' worth of loads, is fastest with
+  // two vectors per lane and proportionally more waves.
   if (nvec <= 64) SK_RMS_CASE(1, 1);
   else if (nvec <= 128) SK_RMS_CASE(1, 2);
-  else if (nvec <= 256) SK_RMS_CASE(1, 4);
-  else if (nvec <= 512) SK_RMS_CASE(2, 4);
-  else if (nvec <= 1024) SK_RMS_CASE(4, 4);
-  else if (nvec <= 2048) SK_RMS_CASE(8, 4);
-  else SK_RMS_CASE(16, 4);
+  else if (FUSED) {
+    if (nvec <= 256) SK_RMS_CASE(2, 2);
+    else if (nvec <= 512) SK_RMS_CASE(4, 2);
+    else if (nvec <= 1024) SK_RMS_CASE(8, 2);
+    else if (nvec <= 2048) SK_RMS_CASE(16, 2);
+    else SK_RMS_CASE(16, 4);
+  } else {
+    if (nvec <= 256) SK_RMS_CASE(1, 4);
+    else if (nvec <= 512) SK_RMS_CASE(1, 8);
+    else if (nvec <= 1024) SK_RMS_CASE(4, 4);
+    else if (nvec <= 2048) SK_RMS_CASE(8, 4);
+    else SK_RMS_CASE(16, 4);
+  }
 #undef SK_RMS_CASE
   return launch_status();
 }

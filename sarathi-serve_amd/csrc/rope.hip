@@ -25,7 +25,6 @@
 
 namespace sarathi_hip {
 
-constexpr int kMaxGridY = 65535;
 constexpr uint32_t kClipped = 0x80000000u;  // byte offset beyond any row: access is dropped
 
 struct RopeArgs {
@@ -44,39 +43,63 @@ struct RopeArgs {
 
 template <int DT> SK_DEV float mul_r(float a, float b) { return rnd<DT>(a * b); }
 
-// slots = 16-byte slots per head (NeoX: of the x half; GPT-J: of the rotated span);
-// slot_shift = log2(slots) or -1 when slots is not a power of two.
+// Kernel arguments are laid out so that everything the first loads need sits in
+// the first 56 bytes, which the hardware preloads into scalar registers at wave
+// launch: the wave can issue its q/k loads without waiting for an argument fetch,
+// and only then fetches the token's position and, from it, the cos/sin row.
+//   geom  = head_bytes | embed_bytes << 16          (bytes of one head / of rot_dim/2)
+//   heads = num_heads | num_kv_heads << 12 | slot_shift << 24
+// slot_shift = log2(16-byte slots per head); NeoX counts the slots of the x half,
+// GPT-J those of the whole rotated span.
 template <int DT, bool NEOX>
-__global__ __launch_bounds__(64) void rope_seg_kernel(RopeArgs a, int64_t tok0, int q_blocks,
-                                                      int slots, int slot_shift) {
+__global__ __launch_bounds__(64) void rope_seg_kernel(
+    const int64_t* __restrict__ positions, void* query, void* key, const void* __restrict__ cache,
+    int64_t q_stride_bytes, int64_t k_stride_bytes, uint32_t geom, uint32_t heads) {
   constexpr int N = VecElems<DT>::value;
-  constexpr int EB = ElemBytes<DT>::value;
-  const int64_t tok = tok0 + (int64_t)blockIdx.z * kMaxGridY + blockIdx.y;
+  const uint32_t head_bytes = geom & 0xffffu, embed_bytes = geom >> 16;
+  const int num_heads = heads & 0xfffu, num_kv_heads = (heads >> 12) & 0xfffu;
+  const int slot_shift = heads >> 24;
+  const int q_blocks = ((num_heads << slot_shift) + 63) >> 6;
+  const int64_t tok = (int64_t)blockIdx.z * kMaxGridY + blockIdx.y;
   const bool is_q = (int)blockIdx.x < q_blocks;  // uniform over the wave
   const int item = ((int)blockIdx.x - (is_q ? 0 : q_blocks)) * 64 + (int)threadIdx.x;
-  const int nheads = is_q ? a.num_heads : a.num_kv_heads;
-  int h, slot;
-  if (slot_shift >= 0) {
-    h = item >> slot_shift;
-    slot = item & (slots - 1);
-  } else {
-    h = item / slots;
-    slot = item - h * slots;
-  }
-  const uint32_t embed_bytes = (uint32_t)(a.rot_dim >> 1) * EB;
-  char* base = reinterpret_cast<char*>(is_q ? a.query : a.key) +
-               tok * (is_q ? a.q_stride : a.k_stride) * EB;
-  const rsrc_t rd = make_rsrc(base, (uint32_t)nheads * a.head_size * EB);
-  const rsrc_t rc = make_rsrc(
-      reinterpret_cast<const char*>(a.cache) + a.positions[tok] * a.rot_dim * EB, 2 * embed_bytes);
-  const uint32_t xoff = h < nheads ? (uint32_t)h * a.head_size * EB + slot * 16u : kClipped;
+  const int nheads = is_q ? num_heads : num_kv_heads;
+  const int h = item >> slot_shift;
+  const uint32_t slot = item & ((1 << slot_shift) - 1);
+  char* base = reinterpret_cast<char*>(is_q ? query : key) +
+               tok * (is_q ? q_stride_bytes : k_stride_bytes);
+  const rsrc_t rd = make_rsrc(base, (uint32_t)nheads * head_bytes);
+  const uint32_t xoff = h < nheads ? (uint32_t)h * head_bytes + slot * 16u : kClipped;
 
+  u32x4 xr, yr;
+  xr = buf_load16<kStreamLoad>(rd, xoff);
+  if constexpr (NEOX) yr = buf_load16<kStreamLoad>(rd, xoff + embed_bytes);
+  // keep the position fetch (and everything hanging off it) behind the loads above
+  __builtin_amdgcn_sched_barrier(0);
+  const rsrc_t rc = make_rsrc(
+      reinterpret_cast<const char*>(cache) + positions[tok] * (int64_t)(2 * embed_bytes),
+      2 * embed_bytes);
+
+  u32x4 cr, sr;
   if constexpr (NEOX) {
-    Vec<DT> x, y, c, s, ox, oy;
-    x.unpack(buf_load16<kStreamLoad>(rd, xoff));
-    y.unpack(buf_load16<kStreamLoad>(rd, xoff + embed_bytes));
-    c.unpack(buf_load16<kCached>(rc, slot * 16u));
-    s.unpack(buf_load16<kCached>(rc, embed_bytes + slot * 16u));
+    cr = buf_load16<kCached>(rc, slot * 16u);
+    sr = buf_load16<kCached>(rc, embed_bytes + slot * 16u);
+  } else {
+    const u32x2 c2 = buf_load8<kCached>(rc, slot * 8u);
+    const u32x2 s2 = buf_load8<kCached>(rc, embed_bytes + slot * 8u);
+    cr = (u32x4){c2.x, c2.y, 0, 0};
+    sr = (u32x4){s2.x, s2.y, 0, 0};
+  }
+  // all four loads are in flight before the first result is waited for
+  __builtin_amdgcn_sched_barrier(0);
+
+  Vec<DT> x, c, s;
+  x.unpack(xr);
+  c.unpack(cr);
+  s.unpack(sr);
+  if constexpr (NEOX) {
+    Vec<DT> y, ox, oy;
+    y.unpack(yr);
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       ox.f[i] = mul_r<DT>(x.f[i], c.f[i]) - mul_r<DT>(y.f[i], s.f[i]);
@@ -85,12 +108,7 @@ __global__ __launch_bounds__(64) void rope_seg_kernel(RopeArgs a, int64_t tok0, 
     buf_store16<kStreamStore>(rd, xoff, ox.pack());
     buf_store16<kStreamStore>(rd, xoff + embed_bytes, oy.pack());
   } else {
-    Vec<DT> x, c, s, o;
-    x.unpack(buf_load16<kStreamLoad>(rd, xoff));
-    const u32x2 c2 = buf_load8<kCached>(rc, slot * 8u);
-    const u32x2 s2 = buf_load8<kCached>(rc, embed_bytes + slot * 8u);
-    c.unpack((u32x4){c2.x, c2.y, 0, 0});
-    s.unpack((u32x4){s2.x, s2.y, 0, 0});
+    Vec<DT> o;
 #pragma unroll
     for (int i = 0; i < N / 2; ++i) {
       const float xe = x.f[2 * i], ye = x.f[2 * i + 1];
@@ -145,22 +163,35 @@ static int launch_rope(const RopeArgs& a, hipStream_t st) {
     return launch_status();
   }
   const int slots = span / N;
-  int slot_shift = -1;
-  if ((slots & (slots - 1)) == 0) {
-    slot_shift = 0;
-    while ((1 << slot_shift) < slots) ++slot_shift;
+  int slot_shift = 0;
+  while ((1 << slot_shift) < slots) ++slot_shift;
+  const int64_t head_bytes = (int64_t)a.head_size * EB;
+  // the packed-argument kernel needs power-of-two slots and fields that fit their bit widths
+  const bool packable = (1 << slot_shift) == slots && head_bytes < 65536 && embed * EB < 65536 &&
+                        a.num_heads < 4096 && a.num_kv_heads < 4096;
+  if (!packable) {
+    hipLaunchKernelGGL((rope_generic_kernel<DT, NEOX>), dim3((unsigned)a.num_tokens), dim3(256),
+                       0, st, a);
+    return launch_status();
   }
+  const uint32_t geom = (uint32_t)head_bytes | ((uint32_t)(embed * EB) << 16);
+  const uint32_t heads =
+      (uint32_t)a.num_heads | ((uint32_t)a.num_kv_heads << 12) | ((uint32_t)slot_shift << 24);
   const int64_t q_blocks = ((int64_t)a.num_heads * slots + 63) / 64;
   const int64_t k_blocks = ((int64_t)a.num_kv_heads * slots + 63) / 64;
-  if (q_blocks + k_blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
   const unsigned gx = (unsigned)(q_blocks + k_blocks);
+  const int64_t qsb = a.q_stride * EB, ksb = a.k_stride * EB;
+  // tokens above 65535 spill into grid.z; the ragged remainder is launched apart
   const int64_t full_z = a.num_tokens / kMaxGridY, rem = a.num_tokens % kMaxGridY;
   if (full_z > 0)
     hipLaunchKernelGGL((rope_seg_kernel<DT, NEOX>), dim3(gx, kMaxGridY, (unsigned)full_z), dim3(64),
-                       0, st, a, (int64_t)0, (int)q_blocks, slots, slot_shift);
-  if (rem > 0)
-    hipLaunchKernelGGL((rope_seg_kernel<DT, NEOX>), dim3(gx, (unsigned)rem, 1), dim3(64), 0, st, a,
-                       full_z * kMaxGridY, (int)q_blocks, slots, slot_shift);
+                       0, st, a.positions, a.query, a.key, a.cache, qsb, ksb, geom, heads);
+  if (rem > 0) {
+    const int64_t t0 = full_z * kMaxGridY;
+    hipLaunchKernelGGL((rope_seg_kernel<DT, NEOX>), dim3(gx, (unsigned)rem, 1), dim3(64), 0, st,
+                       a.positions + t0, reinterpret_cast<char*>(a.query) + t0 * qsb,
+                       reinterpret_cast<char*>(a.key) + t0 * ksb, a.cache, qsb, ksb, geom, heads);
+  }
   return launch_status();
 }
 

@@ -111,10 +111,17 @@ template <int DT> struct Vec {
 //                        than nt alone on MI355X copies
 //   kCached      0       rows that are re-read by many workgroups (weights,
 //                        cos/sin cache)
+// The two streaming policies can be overridden at compile time for tuning runs.
+#ifndef SARATHI_STREAM_LOAD_POLICY
+#define SARATHI_STREAM_LOAD_POLICY 2
+#endif
+#ifndef SARATHI_STREAM_STORE_POLICY
+#define SARATHI_STREAM_STORE_POLICY (2 | 16)
+#endif
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 constexpr int kCached = 0;
-constexpr int kStreamLoad = 2;
-constexpr int kStreamStore = 2 | 16;
+constexpr int kStreamLoad = SARATHI_STREAM_LOAD_POLICY;
+constexpr int kStreamStore = SARATHI_STREAM_STORE_POLICY;
 
 SK_DEV rsrc_t make_rsrc(const void* base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);

@@ -57,9 +57,11 @@ def test_fused_add_rms_norm_matches_oracle(ops, dev, dtype, T, H):
     assert_close_dtype(gx, wx, **_tol(dtype))
 
 
-def test_fused_add_equals_add_then_norm_bitwise(ops, dev):
-    """fused(x, r) == (r' = x + r in bf16; rms_norm(r')) bit for bit, using the library's own
-    rms_norm: the fusion changes traffic, not arithmetic."""
+def test_fused_add_equals_add_then_norm(ops, dev):
+    """fused(x, r) == (r' = x + r in bf16; rms_norm(r')) using the library's own rms_norm: the
+    fusion changes traffic, not arithmetic.  The residual is bit-exact; the normed output may
+    differ in a rare last place because the two kernels split a row over lanes differently and
+    therefore add the squares in a different order."""
     g = gen(3)
     T, H = 2304, 4096
     x, r = randn((T, H), g).to(dev), randn((T, H), g).to(dev)
@@ -68,7 +70,8 @@ def test_fused_add_equals_add_then_norm_bitwise(ops, dev):
     want = torch.empty_like(z)
     ops.layernorm_ops.rms_norm(want, z, w, 1e-5)
     ops.layernorm_ops.fused_add_rms_norm(x, r, w, 1e-5)
-    assert torch.equal(r, z) and torch.equal(x, want)
+    assert torch.equal(r, z)
+    assert_close_dtype(x, want, max_mismatch_frac=1e-4)
 
 
 def test_rms_norm_row_strides(ops, dev):
