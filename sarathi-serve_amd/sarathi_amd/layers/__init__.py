@@ -1,0 +1,13 @@
+"""Counterparts of the reference's Python layer classes that sit directly on the ops
+(sarathi/model_executor/layers/{layernorm,activation,rotary_embedding}.py and the routing helpers of
+layers/fused_moe/fused_moe.py).  Same class / function names and call signatures, so model code written
+against the reference's layers runs unchanged; the bodies call this package's HIP ops."""
+from .activation import FastGELU, NewGELU, SiluAndMul, get_act_fn
+from .moe_routing import fused_topk, moe_align_block_size
+from .norm import RMSNorm
+from .rotary import (DynamicNTKScalingRotaryEmbedding, LinearScalingRotaryEmbedding,
+                     RotaryEmbedding, YaRNScalingRotaryEmbedding, get_rope)
+
+__all__ = ["RMSNorm", "SiluAndMul", "NewGELU", "FastGELU", "get_act_fn", "RotaryEmbedding",
+           "LinearScalingRotaryEmbedding", "DynamicNTKScalingRotaryEmbedding",
+           "YaRNScalingRotaryEmbedding", "get_rope", "fused_topk", "moe_align_block_size"]

@@ -1,0 +1,41 @@
+"""MoE routing helpers (reference: layers/fused_moe/fused_moe.py:151-204 and :346-373)."""
+from typing import Tuple
+
+import torch
+
+from .. import moe_ops
+
+
+def fused_topk(hidden_states: torch.Tensor, gating_output: torch.Tensor, topk: int,
+               renormalize: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Softmax over the experts and top-k per token.  Returns (topk_weights f32 [M, topk],
+    topk_ids i32 [M, topk]).  With ``renormalize`` the weights of a token are divided by their sum,
+    inside the same kernel (the reference does it with a separate tensor divide)."""
+    assert hidden_states.shape[0] == gating_output.shape[0], "Number of tokens mismatch"
+    M = hidden_states.shape[0]
+    dev = hidden_states.device
+    topk_weights = torch.empty((M, topk), dtype=torch.float32, device=dev)
+    topk_ids = torch.empty((M, topk), dtype=torch.int32, device=dev)
+    token_expert_indices = torch.empty((M, topk), dtype=torch.int32, device=dev)
+    logits = gating_output if gating_output.dtype == torch.float32 else gating_output.float()
+    op = moe_ops.topk_softmax_renorm if renormalize else moe_ops.topk_softmax
+    op(topk_weights, topk_ids, token_expert_indices, logits.contiguous())
+    return topk_weights, topk_ids
+
+
+def moe_align_block_size(topk_ids: torch.Tensor, block_size: int,
+                         num_experts: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Sorts the flat (token, k) slots by expert and pads every expert's run to a multiple of
+    ``block_size``.  Returns (sorted_token_ids, expert_ids, num_tokens_post_padded) with the buffer
+    sizes of the reference wrapper; padding slots hold ``topk_ids.numel()`` (written by the kernel
+    itself, so there is no separate fill)."""
+    numel = topk_ids.numel()
+    max_padded = numel + num_experts * (block_size - 1)
+    dev = topk_ids.device
+    sorted_ids = torch.empty((max_padded,), dtype=torch.int32, device=dev)
+    expert_ids = torch.empty(((max_padded + block_size - 1) // block_size,), dtype=torch.int32,
+                             device=dev)
+    num_tokens_post_pad = torch.empty((1,), dtype=torch.int32, device=dev)
+    moe_ops.moe_align_block_size_filled(topk_ids.contiguous(), num_experts, block_size, sorted_ids,
+                                        expert_ids, num_tokens_post_pad)
+    return sorted_ids, expert_ids, num_tokens_post_pad

@@ -1,0 +1,163 @@
+"""GPU: the benchmark configurations at their full sizes, checked against the oracle on a random
+sample of token rows (every op here is per-token, so a row of the full-size output must equal the
+oracle run on that row alone), and HIP-graph capture of the layer chain."""
+import pytest
+import torch
+
+from helpers import (THETA_LLAMA3, assert_close_dtype, cos_sin_cache, gen, hybrid_positions, randn)
+from oracle import c_oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _chain_gpu(ops, s):
+    ops.layernorm_ops.fused_add_rms_norm(s["x"], s["res"], s["w1"], 1e-5)
+    ops.pos_encoding_ops.rotary_embedding(s["pos"], s["q"], s["k"], s["D"], s["cache"], True)
+    ops.activation_ops.silu_and_mul(s["act"], s["gate_up"])
+    ops.layernorm_ops.fused_add_rms_norm(s["x"], s["res"], s["w2"], 1e-5)
+
+
+def _make(T, prefill, H, nq, nkv, D, dff, seed, dev):
+    """Device-side random inputs (the sampled rows are copied back for the oracle)."""
+    torch.manual_seed(seed)
+    g = gen(seed)
+    bf = torch.bfloat16
+    mk = lambda *shape: torch.randn(shape, device=dev, dtype=torch.float32).to(bf)  # noqa: E731
+    s = {"D": D}
+    s["x"], s["res"] = mk(T, H), mk(T, H)
+    s["w1"] = randn((H,), g, mean=1.0, std=0.1).to(dev)
+    s["w2"] = randn((H,), g, mean=1.0, std=0.1).to(dev)
+    s["qkv"] = mk(T, (nq + 2 * nkv) * D)
+    s["q"], s["k"], s["v"] = s["qkv"].split([nq * D, nkv * D, nkv * D], dim=-1)
+    s["pos"] = hybrid_positions(T, prefill, g).to(dev)
+    s["cache"] = cos_sin_cache(8192, D, THETA_LLAMA3, bf).to(dev)
+    s["gate_up"] = mk(T, 2 * dff)
+    s["act"] = torch.empty((T, dff), dtype=bf, device=dev)
+    return s
+
+
+@pytest.mark.parametrize("name,T,prefill,H,nq,nkv,D,dff", [
+    ("llama3-8b hybrid batch", 2304, 2048, 4096, 32, 8, 128, 14336),
+    ("llama3-70b chain", 4608, 4096, 8192, 64, 8, 128, 28672),
+])
+def test_full_size_chain_rows_match_oracle(ops, dev, name, T, prefill, H, nq, nkv, D, dff):
+    s = _make(T, prefill, H, nq, nkv, D, dff, 4, dev)
+    g = gen(5)
+    rows = torch.cat((torch.tensor([0, prefill - 1, prefill, T - 1]),
+                      torch.randint(0, T, (60,), generator=g))).unique()
+    rd = rows.to(dev)
+    # oracle on the sampled rows only (taken before the in-place ops run)
+    ox, ores = s["x"][rd].cpu(), s["res"][rd].cpu()
+    oqkv = s["qkv"][rd].cpu()
+    ogu = s["gate_up"][rd].cpu()
+    w1, w2, cache, pos = s["w1"].cpu(), s["w2"].cpu(), s["cache"].cpu(), s["pos"][rd].cpu()
+    v_before = s["v"].clone()
+    _chain_gpu(ops, s)
+    torch.cuda.synchronize()
+
+    c_oracle.fused_add_rms_norm(ox, ores, w1, 1e-5)
+    oq, ok, _ = oqkv.split([nq * D, nkv * D, nkv * D], dim=-1)
+    c_oracle.rotary_embedding(pos, oq, ok, D, cache, True)
+    oact = torch.empty((rows.numel(), dff), dtype=torch.bfloat16)
+    c_oracle.silu_and_mul(oact, ogu)
+    x1 = ox.clone()                       # after the first norm
+    c_oracle.fused_add_rms_norm(ox, ores, w2, 1e-5)
+
+    assert torch.equal(s["qkv"][rd].cpu(), oqkv), name            # rope: bit-exact
+    assert torch.equal(s["v"], v_before)                          # v part of the packed buffer untouched
+    assert_close_dtype(s["act"][rd], oact)
+    # the second fused norm consumed the first one's (tolerance-level) output, so compare it with
+    # the oracle fed the oracle's own first-norm output: same tolerance, few extra flips
+    assert_close_dtype(s["res"][rd], ores, max_mismatch_frac=2e-2)
+    assert_close_dtype(s["x"][rd], ox, max_mismatch_frac=2e-2)
+    del x1
+
+
+def test_mixtral_routing_full_size(ops, dev):
+    """Benchmark configuration 4: logits fp32 [4096, 8], top-2 (renormalised), align block 64."""
+    g = gen(3)
+    M, E, k, B = 4096, 8, 2, 64
+    gating = torch.randn((M, E), generator=g, dtype=torch.float32)
+    ww, wi, ws = torch.empty((M, k)), torch.empty((M, k), dtype=torch.int32), torch.empty((M, k), dtype=torch.int32)
+    c_oracle.topk_softmax(ww, wi, ws, gating)
+    gw = torch.empty((M, k), dtype=torch.float32, device=dev)
+    gi = torch.empty((M, k), dtype=torch.int32, device=dev)
+    gs = torch.empty((M, k), dtype=torch.int32, device=dev)
+    ops.moe_ops.topk_softmax_renorm(gw, gi, gs, gating.to(dev))
+    assert torch.equal(gi.cpu(), wi) and torch.equal(gs.cpu(), ws)
+    assert torch.allclose(gw.cpu(), ww / ww.sum(-1, keepdim=True), rtol=0, atol=1e-6)
+    n = M * k + E * (B - 1)
+    sg = torch.empty((n,), dtype=torch.int32, device=dev)
+    eg = torch.full(((n + B - 1) // B,), -1, dtype=torch.int32, device=dev)
+    pg = torch.empty((1,), dtype=torch.int32, device=dev)
+    ops.moe_ops.moe_align_block_size_filled(gi, E, B, sg, eg, pg)
+    sw = torch.full((n,), M * k, dtype=torch.int32)
+    ew = torch.full(((n + B - 1) // B,), -1, dtype=torch.int32)
+    pw = torch.zeros((1,), dtype=torch.int32)
+    c_oracle.moe_align_block_size(wi, E, B, sw, ew, pw)
+    nb = int(pw.item()) // B
+    assert n == 8696 and eg.numel() == 136
+    assert torch.equal(sg.cpu(), sw) and torch.equal(pg.cpu(), pw) and torch.equal(eg.cpu()[:nb], ew[:nb])
+    assert bool((eg.cpu()[nb:] == -1).all())
+
+
+def test_chain_and_routing_under_hip_graph_capture(ops, dev):
+    """The ops allocate nothing and launch fixed shapes, so a captured graph replays them.  Each
+    replay is checked against an eager run on the same inputs, with eager work and synchronisation
+    between the replays."""
+    T, H, nq, nkv, D, dff = 512, 4096, 32, 8, 128, 14336
+    s = _make(T, 448, H, nq, nkv, D, dff, 6, dev)
+    M, E, k, B = 1024, 8, 2, 64
+    g = gen(7)
+    gating = torch.randn((M, E), generator=g, dtype=torch.float32).to(dev)
+    tw = torch.empty((M, k), dtype=torch.float32, device=dev)
+    ti = torch.empty((M, k), dtype=torch.int32, device=dev)
+    ts = torch.empty((M, k), dtype=torch.int32, device=dev)
+    n = M * k + E * (B - 1)
+    sg = torch.empty((n,), dtype=torch.int32, device=dev)
+    eg = torch.zeros(((n + B - 1) // B,), dtype=torch.int32, device=dev)
+    pg = torch.empty((1,), dtype=torch.int32, device=dev)
+    keys = ("x", "res", "qkv", "gate_up")
+    init = {kk: s[kk].clone() for kk in keys}
+
+    def run_all():
+        _chain_gpu(ops, s)
+        ops.moe_ops.topk_softmax(tw, ti, ts, gating)
+        ops.moe_ops.moe_align_block_size_filled(ti, E, B, sg, eg, pg)
+
+    def reset():
+        for kk in keys:
+            s[kk].copy_(init[kk])
+
+    def snapshot():
+        return [t.clone() for t in (s["x"], s["res"], s["qkv"], s["act"], tw, ti, ts, sg, eg, pg)]
+
+    reset()
+    run_all()
+    torch.cuda.synchronize()
+    want = snapshot()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):          # warm-up on the capture stream, as torch requires
+        reset()
+        run_all()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    reset()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        run_all()
+    for it in range(4):
+        reset()
+        for t in (s["act"], tw, sg):
+            t.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = snapshot()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b), "replay %d differs from the eager run" % it
+        # unrelated eager work between replays
+        _ = (s["gate_up"].float().sum() + gating.sum()).item()

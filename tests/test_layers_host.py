@@ -1,0 +1,114 @@
+"""Host-side logic of the layer counterparts, without a GPU: the cos || sin table builders of the
+rotary variants (closed forms and reductions between variants), the factory, the activation
+registry."""
+import math
+
+import pytest
+import torch
+
+from helpers import cos_sin_cache
+
+
+@pytest.fixture(scope="module")
+def L(ops):
+    from sarathi_amd import layers
+    return layers
+
+
+def _rope(L, scaling=None, D=64, max_pos=256, base=10000, dtype=torch.float32):
+    return L.get_rope(D, D, max_pos, base, True, scaling, device="cpu", dtype=dtype)
+
+
+def test_default_table_closed_form(L):
+    r = _rope(L)
+    c = r.cos_sin_cache
+    assert c.shape == (256, 64) and c.dtype == torch.float32
+    for p, i in [(0, 0), (1, 0), (17, 5), (255, 31), (100, 16)]:
+        ang = p / (10000 ** (2 * i / 64))
+        assert abs(c[p, i].item() - math.cos(ang)) < 2e-5 and abs(c[p, 32 + i].item() - math.sin(ang)) < 2e-5
+    assert torch.equal(c[0, :32], torch.ones(32)) and torch.equal(c[0, 32:], torch.zeros(32))
+    # the bf16 table of the benchmark configuration is what the tests' helper builds
+    big = L.get_rope(128, 128, 8192, 500000, True, None, device="cpu", dtype=torch.bfloat16)
+    assert torch.equal(big.cos_sin_cache, cos_sin_cache(8192, 128, 500000.0, torch.bfloat16))
+
+
+def test_linear_scaling_reduces_to_default_at_multiples(L):
+    base = _rope(L).cos_sin_cache
+    lin = _rope(L, {"type": "linear", "factor": 4.0})
+    assert isinstance(lin, L.LinearScalingRotaryEmbedding)
+    assert lin.cos_sin_cache.shape == (1024, 64)
+    assert torch.allclose(lin.cos_sin_cache[0::4], base, atol=1e-6)     # position 4p uses angle p
+    assert not torch.allclose(lin.cos_sin_cache[:256], base, atol=1e-3)
+
+
+def test_dynamic_ntk_closed_form(L):
+    f = 2.0
+    dyn = _rope(L, {"type": "dynamic", "factor": f})
+    assert isinstance(dyn, L.DynamicNTKScalingRotaryEmbedding)
+    assert dyn.cos_sin_cache.shape == (512, 64)
+    new_base = 10000 * ((f * 512 / 256) - (f - 1)) ** (64 / 62)
+    for p, i in [(3, 1), (500, 20), (77, 31)]:
+        ang = p / (new_base ** (2 * i / 64))
+        assert abs(dyn.cos_sin_cache[p, i].item() - math.cos(ang)) < 5e-5
+    one = _rope(L, {"type": "dynamic", "factor": 1.0})
+    assert torch.equal(one.cos_sin_cache, _rope(L).cos_sin_cache)       # factor 1: base unchanged
+
+
+def test_yarn_properties(L):
+    f, D, orig = 4.0, 64, 256
+    sc = {"type": "yarn", "factor": f, "original_max_position_embeddings": orig}
+    y = L.get_rope(D, D, int(orig * f), 10000, True, sc, device="cpu", dtype=torch.float32)
+    assert isinstance(y, L.YaRNScalingRotaryEmbedding)
+    assert y.cos_sin_cache.shape == (1024, 64)
+    assert abs(y.mscale - (0.1 * math.log(f) + 1.0)) < 1e-12
+    inv = y._compute_inv_freq(f)
+    plain = 1.0 / (10000 ** (torch.arange(0, D, 2, dtype=torch.float) / D))
+    from sarathi_amd.layers.rotary import yarn_correction_range
+    low, high = yarn_correction_range(32, 1, D, 10000, orig)
+    assert 0 <= low < high <= D - 1
+    assert torch.allclose(inv[: low + 1], plain[: low + 1])             # fast dims keep their frequency
+    assert torch.allclose(inv[high:], plain[high:] / f)                 # slow dims are interpolated
+    mid = inv[low + 1: high]
+    assert bool((mid < plain[low + 1: high]).all()) and bool((mid > plain[low + 1: high] / f).all())
+    # row 0: cos = mscale, sin = 0
+    assert torch.allclose(y.cos_sin_cache[0, :32], torch.full((32,), y.mscale))
+    assert torch.equal(y.cos_sin_cache[0, 32:], torch.zeros(32))
+    # factor 1 is the plain table
+    one = L.get_rope(D, D, orig, 10000, True, {"type": "yarn", "factor": 1.0,
+                                               "original_max_position_embeddings": orig},
+                     device="cpu", dtype=torch.float32)
+    assert torch.allclose(one.cos_sin_cache, _rope(L, None, D, orig).cos_sin_cache, atol=1e-6)
+    # extra keyword arguments are routed through the factory
+    y2 = L.get_rope(D, D, int(orig * f), 10000, True, dict(sc, attn_factor=2.0, beta_fast=16),
+                    device="cpu", dtype=torch.float32)
+    assert abs(y2.mscale - 2.0 * y.mscale) < 1e-12 and y2.beta_fast == 16
+
+
+def test_factory_errors_and_dtype(L):
+    with pytest.raises(ValueError):
+        _rope(L, {"type": "ntk-by-parts", "factor": 2.0})
+    with pytest.raises(AssertionError):
+        L.get_rope(64, 64, 1000, 10000, True, {"type": "yarn", "factor": 4.0,
+                                               "original_max_position_embeddings": 256}, device="cpu")
+    assert _rope(L, dtype=torch.float16).cos_sin_cache.dtype == torch.float16
+    prev = torch.get_default_dtype()
+    try:
+        torch.set_default_dtype(torch.bfloat16)      # the reference casts to the default dtype
+        assert L.get_rope(64, 64, 32, 10000, True, None, device="cpu").cos_sin_cache.dtype == torch.bfloat16
+    finally:
+        torch.set_default_dtype(prev)
+
+
+def test_activation_registry(L):
+    assert isinstance(L.get_act_fn("gelu_new"), L.NewGELU)
+    assert isinstance(L.get_act_fn("GELU_FAST"), L.FastGELU)
+    assert isinstance(L.get_act_fn("relu"), torch.nn.ReLU)
+    assert L.get_act_fn("gelu_pytorch_tanh").approximate == "tanh"
+    with pytest.raises(ValueError):
+        L.get_act_fn("swish")
+
+
+def test_rmsnorm_module_state(L):
+    n = L.RMSNorm(128, eps=1e-5, norm_name="input_layernorm", layer_id=10)
+    assert n.weight.shape == (128,) and bool((n.weight == 1).all())
+    assert n.variance_epsilon == 1e-5 and n.norm_name == "input_layernorm" and n.layer_id == 10
