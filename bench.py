@@ -57,6 +57,13 @@ BYTES["moe_align_block_size"] = MOE_T * MOE_K * 4 + _moe_sorted * 4 + 4 * (
     (_moe_sorted + MOE_B - 1) // MOE_B) + 4
 
 
+# HBM bytes per silu_and_mul launch at this shape as measured with rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (two runs), each counter scaled by what it reads for a plain 256 MiB copy:
+# (64522.9 KiB * 1.9997 + 64512.0 KiB * 1.0000) * 1024.  Counters cannot be read from inside
+# this script; the summary with the commands is profiles/kernels_llama3_8b_t2304_pmc_fetch_write.txt.
+SILU_MEASURED_HBM_BYTES = 198186464
+
+
 def make_set(torch, g, dev, cache_cpu):
     """One independent set of step inputs (seeded on the CPU, fp32 draw -> bf16)."""
     from helpers import hybrid_positions, randn
@@ -84,9 +91,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a 256 MiB plain copy (counter calibration for --pmc runs)")
-    ap.add_argument("--traffic", type=float, default=None,
-                    help="measured HBM bytes per silu_and_mul launch (from a --pmc run), reported "
-                         "verbatim as roofline.traffic")
+    ap.add_argument("--traffic", type=float, default=SILU_MEASURED_HBM_BYTES,
+                    help="measured HBM bytes per silu_and_mul launch, reported verbatim as "
+                         "roofline.traffic (default: the figure of the committed rocprofv3 --pmc "
+                         "summary under profiles/)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this op library runs on one GPU; --gpus must be 1 "
@@ -257,7 +265,7 @@ def main():
         t_start = time.perf_counter()
         cpu_step()
         one = time.perf_counter() - t_start
-        reps = max(3, min(50, int(12.0 / max(one, 1e-3))))
+        reps = max(3, min(2000, int(12.0 / max(one, 1e-3))))      # about 12 s of CPU work
         times = []
         for _ in range(reps):
             t_start = time.perf_counter()

@@ -138,12 +138,28 @@ int sarathi_topk_softmax(float* topk_weights, int32_t* topk_indices,
  * expert_ids entries at or above num_tokens_post_pad / block_size are left
  * untouched.  Ids outside [0, num_experts) are skipped (the reference's
  * behaviour for them is undefined).
+ *
+ * `workspace` is optional device scratch of `workspace_bytes` bytes (4-byte
+ * aligned, contents irrelevant on entry and exit).  Without it, or when it is
+ * smaller than sarathi_moe_align_workspace_bytes() asks for, the sort runs in a
+ * single workgroup, which is the fastest path up to ~16 K ids; with it, larger
+ * inputs are spread over the whole GPU in three launches.  Results are
+ * identical either way.
  */
 int sarathi_moe_align_block_size(const void* topk_ids, int id_dtype, int64_t numel,
                                  int num_experts, int block_size, int32_t* sorted_token_ids,
                                  int64_t sorted_len, int32_t* expert_ids,
                                  int64_t expert_ids_len, int32_t* num_tokens_post_pad,
-                                 int fill_pad, void* stream);
+                                 int fill_pad, void* workspace, int64_t workspace_bytes,
+                                 void* stream);
+
+/*
+ * Scratch bytes sarathi_moe_align_block_size can make use of for this input
+ * size; 0 when the single-workgroup path will be taken anyway.  The reference
+ * allocates a workspace in the same way for topk_softmax
+ * (csrc/moe_topk_softmax_kernels.cu:486-492).
+ */
+int64_t sarathi_moe_align_workspace_bytes(int64_t numel, int num_experts);
 
 #ifdef __cplusplus
 }

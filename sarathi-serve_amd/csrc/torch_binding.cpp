@@ -7,7 +7,8 @@
 // rank, inner contiguity; (b) makes the tensors' device current and looks up
 // torch's current HIP stream for it; (c) forwards raw pointers, sizes and
 // strides to the C ABI of include/sarathi_ops.h and turns a non-zero status
-// into a RuntimeError.  It never allocates, copies or synchronises.
+// into a RuntimeError.  It never copies or synchronises, and allocates only the scratch
+// tensor that moe_align_block_size uses for inputs above 16 K ids.
 #include <c10/hip/HIPStream.h>
 #include <hip/hip_runtime_api.h>
 #include <torch/extension.h>
@@ -249,11 +250,19 @@ void moe_align_impl(torch::Tensor& topk_ids, int64_t num_experts, int64_t block_
                   block_size <= INT32_MAX,
               op, ": num_experts and block_size must be positive");
   LaunchScope scope(topk_ids);
+  // Large inputs get a scratch tensor from torch's caching allocator (stream-ordered, so it may
+  // be released as soon as the launches are queued), the way the reference's topk_softmax
+  // obtains its workspace (csrc/moe_topk_softmax_kernels.cu:486-492).
+  const int64_t ws_bytes = sarathi_moe_align_workspace_bytes(topk_ids.numel(), (int)num_experts);
+  torch::Tensor workspace;
+  if (ws_bytes > 0)
+    workspace = torch::empty({ws_bytes / 4}, sorted_token_ids.options());
   raise_on(sarathi_moe_align_block_size(
                topk_ids.data_ptr(), id_dtype_code(topk_ids), topk_ids.numel(), (int)num_experts,
                (int)block_size, sorted_token_ids.data_ptr<int32_t>(), sorted_token_ids.numel(),
                experts_ids.data_ptr<int32_t>(), experts_ids.numel(),
-               num_tokens_post_pad.data_ptr<int32_t>(), fill_pad ? 1 : 0, scope.stream),
+               num_tokens_post_pad.data_ptr<int32_t>(), fill_pad ? 1 : 0,
+               ws_bytes > 0 ? workspace.data_ptr() : nullptr, ws_bytes, scope.stream),
            op);
 }
 

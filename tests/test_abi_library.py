@@ -30,7 +30,8 @@ def test_header_declares_the_expected_entry_points():
     names = declared_functions()
     for n in ["sarathi_rms_norm", "sarathi_fused_add_rms_norm", "sarathi_silu_and_mul",
               "sarathi_gelu_new", "sarathi_gelu_fast", "sarathi_rotary_embedding",
-              "sarathi_topk_softmax", "sarathi_moe_align_block_size", "sarathi_ops_abi_version",
+              "sarathi_topk_softmax", "sarathi_moe_align_block_size",
+              "sarathi_moe_align_workspace_bytes", "sarathi_ops_abi_version",
               "sarathi_ops_strerror"]:
         assert n in names
 
@@ -91,12 +92,19 @@ def test_argument_validation_without_gpu(lib):
     assert topk(p, p, p, p, i64(1), ci(2048), ci(1), ci(0), null) == UNSUPPORTED
     assert topk(p, p, p, p, i64(0), ci(8), ci(2), ci(0), null) == OK
     align = lib.sarathi_moe_align_block_size
-    assert align(p, ci(3), i64(4), ci(8), ci(4), null, i64(64), p, i64(16), p, ci(0), null) == INVALID
-    assert align(p, ci(3), i64(4), ci(0), ci(4), p, i64(64), p, i64(16), p, ci(0), null) == INVALID
-    assert align(p, ci(3), i64(4), ci(8), ci(4), p, i64(8), p, i64(16), p, ci(0), null) == INVALID  # sorted too short
-    assert align(p, ci(3), i64(4), ci(8), ci(4), p, i64(64), p, i64(1), p, ci(0), null) == INVALID  # expert_ids too short
-    assert align(p, ci(3), i64(4), ci(4096), ci(4), p, i64(64), p, i64(16), p, ci(0), null) == UNSUPPORTED
-    assert align(p, ci(11), i64(4), ci(8), ci(4), p, i64(64), p, i64(16), p, ci(0), null) == UNSUPPORTED
+    ws = (null, i64(0), null)      # workspace, workspace_bytes, stream
+    assert align(p, ci(3), i64(4), ci(8), ci(4), null, i64(64), p, i64(16), p, ci(0), *ws) == INVALID
+    assert align(p, ci(3), i64(4), ci(0), ci(4), p, i64(64), p, i64(16), p, ci(0), *ws) == INVALID
+    assert align(p, ci(3), i64(4), ci(8), ci(4), p, i64(8), p, i64(16), p, ci(0), *ws) == INVALID  # sorted too short
+    assert align(p, ci(3), i64(4), ci(8), ci(4), p, i64(64), p, i64(1), p, ci(0), *ws) == INVALID  # expert_ids too short
+    assert align(p, ci(3), i64(4), ci(4096), ci(4), p, i64(64), p, i64(16), p, ci(0), *ws) == UNSUPPORTED
+    assert align(p, ci(11), i64(4), ci(8), ci(4), p, i64(64), p, i64(16), p, ci(0), *ws) == UNSUPPORTED
+    wsb = lib.sarathi_moe_align_workspace_bytes
+    wsb.restype = ctypes.c_int64
+    assert wsb(i64(8192), ci(8)) == 0                       # small inputs: single workgroup
+    big = wsb(i64(131072), ci(8))
+    assert big > 0 and big % 4 == 0 and wsb(i64(131072), ci(256)) > big
+    assert wsb(i64(1 << 20), ci(1024)) <= (1024 * 1024 + 1025) * 4
 
 
 def test_front_end_refuses_cpu_tensors_and_bad_shapes(ops):

@@ -135,7 +135,8 @@ def test_moe_align_reference_vectors(ops, dev):
 @pytest.mark.parametrize("T,k,E,B", [(4096, 2, 8, 64), (4096, 2, 8, 16), (4096, 2, 8, 128),
                                      (1, 1, 8, 64), (7, 2, 8, 32), (63, 1, 4, 4), (64, 1, 4, 4),
                                      (65, 3, 16, 1), (1000, 6, 64, 16), (3000, 8, 256, 32),
-                                     (500, 4, 1000, 8), (70000, 2, 8, 64), (16384, 4, 60, 128)])
+                                     (500, 4, 1000, 8), (70000, 2, 8, 64), (16384, 4, 60, 128),
+                                     (8193, 2, 8, 64), (30000, 4, 1000, 8), (65536, 8, 256, 16)])
 def test_moe_align_matches_oracle(ops, dev, T, k, E, B, filled):
     g = gen(T + E)
     ids = torch.randint(0, E, (T, k), generator=g, dtype=torch.int32)
@@ -192,3 +193,34 @@ def test_moe_align_invariants_large(ops, dev):
         assert bool((flat[row] == ge[b]).all())
         assert bool((row[1:] > row[:-1]).all())
     assert bool((gs[n:] == T * k).all())
+
+
+def test_moe_align_workspace_is_optional(ops, dev):
+    """Straight through the C ABI: with no workspace a large input takes the single-workgroup
+    kernel, with one it takes the three-launch path; both give the oracle's result."""
+    import ctypes
+    import os
+    lib = ctypes.CDLL(os.path.join(os.path.dirname(ops.__file__), "lib", "libsarathi_ops_hip.so"))
+    lib.sarathi_moe_align_workspace_bytes.restype = ctypes.c_int64
+    g = gen(13)
+    T, k, E, B = 40000, 2, 64, 32
+    ids = torch.randint(0, E, (T, k), generator=g, dtype=torch.int32)
+    ws, we, wp = _align_bufs(ids.numel(), E, B, "cpu")
+    c_oracle.moe_align_block_size(ids, E, B, ws, we, wp)
+    need = lib.sarathi_moe_align_workspace_bytes(ctypes.c_int64(ids.numel()), ctypes.c_int(E))
+    assert need > 0
+    ids_d = ids.to(dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for ws_bytes in (0, need // 2, need):
+        scratch = torch.empty((max(ws_bytes, 4) // 4,), dtype=torch.int32, device=dev)
+        gs, ge, gp = _align_bufs(ids.numel(), E, B, dev, fill=False)
+        rc = lib.sarathi_moe_align_block_size(
+            ctypes.c_void_p(ids_d.data_ptr()), ctypes.c_int(3), ctypes.c_int64(ids.numel()),
+            ctypes.c_int(E), ctypes.c_int(B), ctypes.c_void_p(gs.data_ptr()),
+            ctypes.c_int64(gs.numel()), ctypes.c_void_p(ge.data_ptr()), ctypes.c_int64(ge.numel()),
+            ctypes.c_void_p(gp.data_ptr()), ctypes.c_int(1),
+            ctypes.c_void_p(scratch.data_ptr() if ws_bytes else None), ctypes.c_int64(ws_bytes),
+            stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        _check_align((gs.cpu(), ge.cpu(), gp.cpu()), (ws, we, wp), B)
