@@ -224,6 +224,23 @@ def main():
     del ops_table
     torch.cuda.empty_cache()
 
+    # ---- context: a plain device-to-device copy that moves the same number of bytes ----
+    # (torch's copy kernel, cold ring).  Half of an op's algorithmic bytes are read and half
+    # written, which is exactly rms_norm's and rotary_embedding's mix; it shows what the memory
+    # system gives a trivial kernel at each size.
+    copy_ref = {}
+    for name in ("rms_norm", "rotary_embedding", "fused_add_rms_norm", "silu_and_mul"):
+        half = BYTES[name] // 2 // 2 * 2
+        n = max(4, int(COLD_FOOTPRINT // BYTES[name]) + 1)
+        pairs = [(torch.empty(half // 2, dtype=torch.bfloat16, device=dev).fill_(1.0),
+                  torch.empty(half // 2, dtype=torch.bfloat16, device=dev)) for _ in range(n)]
+        us = time_op(lambda a: a[1].copy_(a[0]), pairs, args.steps)
+        gbs = 2 * half / us * 1e-3
+        copy_ref[name] = {"bytes": 2 * half, "us": round(us, 3), "GBps": round(gbs, 1),
+                          "frac_of_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        del pairs
+    torch.cuda.empty_cache()
+
     if args.calibrate_copy:
         src = torch.empty((256 << 20) // 2, dtype=torch.bfloat16, device=dev).fill_(1.0)
         dst = torch.empty_like(src)
@@ -303,6 +320,7 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "per_op": per_op,
+        "plain_copy_same_bytes_cold": copy_ref,
     }
     print(json.dumps(out))
 

@@ -161,6 +161,27 @@ int sarathi_moe_align_block_size(const void* topk_ids, int id_dtype, int64_t num
  */
 int64_t sarathi_moe_align_workspace_bytes(int64_t numel, int num_experts);
 
+/*
+ * Grouped expert GEMM that consumes moe_align_block_size's outputs; replaces the
+ * Triton kernel launched by invoke_fused_moe_kernel
+ * (sarathi/model_executor/layers/fused_moe/fused_moe.py:15-148, :207-260).
+ * For every block of block_m consecutive slots of sorted_token_ids (one expert,
+ * expert_ids[block]):  C[slot, :] = A[slot / top_k, :] @ B[expert]^T, fp32
+ * accumulation, times topk_weights[slot] when mul_routed_weight != 0, rounded
+ * to `dtype`.  A [tokens, K] with rows a_row_stride elements apart, B
+ * [E, N, K] K-contiguous with experts b_expert_stride elements apart, C
+ * [num_valid_tokens, N] with rows c_row_stride apart (num_valid_tokens =
+ * tokens * topk; slots holding a larger id are padding and skipped).
+ * block_m must be the block_size moe_align_block_size ran with and one of 32,
+ * 64, 128; dtype bf16 or fp16; K a multiple of 64, N a multiple of 4.
+ */
+int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c, const float* topk_weights,
+                             const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                             const int32_t* num_tokens_post_padded, int64_t num_valid_tokens,
+                             int64_t sorted_len, int64_t n, int64_t k, int64_t a_row_stride,
+                             int64_t b_expert_stride, int64_t c_row_stride, int block_m,
+                             int top_k, int mul_routed_weight, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

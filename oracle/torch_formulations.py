@@ -92,3 +92,50 @@ def moe_align_block_size(topk_ids, num_experts, block_size, sorted_token_ids, ex
     blk_start = torch.arange(nblk, dtype=torch.int64) * block_size
     experts_ids[:nblk] = (torch.searchsorted(cumsum, blk_start, right=True) - 1).to(torch.int32)
     num_tokens_post_pad[0] = int(cumsum[-1])
+
+
+def moe_grouped_gemm(A, B, C, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                     num_valid_tokens, block_m, top_k, mul_routed_weight):
+    """What the reference's Triton fused_moe_kernel computes
+    (sarathi/model_executor/layers/fused_moe/fused_moe.py:84-147): per block of block_m sorted slots,
+    rows A[slot // top_k] times B[expert]^T with fp32 accumulation, optionally times the slot's
+    routing weight (in fp32), cast to the tensor dtype, stored at row `slot` of C."""
+    n_post = int(num_tokens_post_padded.item())
+    Cf = C.view(-1, B.shape[1])
+    wflat = topk_weights.reshape(-1)
+    for blk in range(n_post // block_m):
+        slots = sorted_token_ids[blk * block_m:(blk + 1) * block_m].long()
+        slots = slots[slots < num_valid_tokens]
+        if slots.numel() == 0:
+            continue
+        e = int(expert_ids[blk].item())
+        acc = A[slots // top_k].float() @ B[e].float().t()
+        if mul_routed_weight:
+            acc = acc * wflat[slots].float().unsqueeze(1)
+        Cf[slots] = acc.to(C.dtype)
+
+
+def fused_moe(hidden_states, w1, w2, gating_output, topk, renormalize):
+    """Dense statement of the MoE layer the reference's fused_moe computes (fused_moe.py:411-622),
+    keeping its intermediate tensors in the model dtype: out[t] = sum_j T(w_j * (h_j @ W2[e_j]^T))
+    with h_j = silu_and_mul(T(x_t @ W1[e_j]^T))."""
+    T, _ = hidden_states.shape
+    dt = hidden_states.dtype
+    tw = torch.empty((T, topk), dtype=torch.float32)
+    ti = torch.empty((T, topk), dtype=torch.int32)
+    ts = torch.empty((T, topk), dtype=torch.int32)
+    topk_softmax(tw, ti, ts, gating_output.float())
+    if renormalize:
+        tw = tw / tw.sum(dim=-1, keepdim=True)
+    inter = w1.shape[1] // 2
+    parts = torch.zeros((T, topk, w2.shape[1]), dtype=dt)
+    for e in range(w1.shape[0]):
+        tok, j = torch.nonzero(ti == e, as_tuple=True)
+        if tok.numel() == 0:
+            continue
+        gate_up = (hidden_states[tok].float() @ w1[e].float().t()).to(dt)
+        act = torch.empty((tok.numel(), inter), dtype=dt)
+        silu_and_mul(act, gate_up)
+        down = (act.float() @ w2[e].float().t()) * tw[tok, j].unsqueeze(1)
+        parts[tok, j] = down.to(dt)
+    return parts.sum(dim=1)

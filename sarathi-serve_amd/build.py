@@ -21,7 +21,8 @@ PKG = os.path.join(HERE, "sarathi_amd")
 LIB_DIR = os.path.join(PKG, "lib")
 OBJ_DIR = os.path.join(HERE, "build", "obj")
 
-HIP_SOURCES = ["rms_norm.hip", "gated_act.hip", "rope.hip", "moe_topk.hip", "moe_align.hip"]
+HIP_SOURCES = ["rms_norm.hip", "gated_act.hip", "rope.hip", "moe_topk.hip", "moe_align.hip",
+               "moe_gemm.hip"]
 CXX_SOURCES = ["abi_misc.cpp"]
 
 ABI_LIB = os.path.join(LIB_DIR, "libsarathi_ops_hip.so")

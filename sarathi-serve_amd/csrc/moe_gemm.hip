@@ -1,0 +1,273 @@
+// Grouped expert GEMM for MoE layers on gfx950 (MFMA).
+//
+// Counterpart of the reference's Triton `fused_moe_kernel`
+// (sarathi/model_executor/layers/fused_moe/fused_moe.py:15-148): for every block of BM
+// consecutive slots of sorted_token_ids (all routed to one expert, expert_ids[block]),
+//   C[slot, :] = A[slot / top_k, :] @ B[expert]^T   (fp32 accumulation)
+// optionally scaled by the slot's routing weight, rounded to the tensor dtype
+// and stored at row `slot` of C.  A is [tokens, K], B is [E, N, K] (K
+// contiguous), C is [tokens * top_k, N].  Padding slots (id >= num_valid) and
+// blocks at or beyond num_tokens_post_padded produce nothing.
+//
+// Tiling: a workgroup of four waves owns BM slots x 256 output columns; wave w
+// owns columns [64 w, 64 w + 64) for all BM slots, as 32x32 MFMA tiles
+// (v_mfma_f32_32x32x16 bf16 / f16, 16 deep).  The MFMA "A" operand is fed with
+// WEIGHT rows and the "B" operand with TOKEN rows, so a lane ends up holding
+// four consecutive output columns of one token per accumulator quad and the
+// epilogue writes 8-byte pieces of C rows.
+//   weights  never shared between waves: each lane loads its 16-byte operand
+//            pieces straight from global memory (buffer loads on the expert's
+//            matrix, clipped at N rows), one K-step (64) ahead of their use;
+//   tokens   shared by the four waves: gathered once per K-step into LDS
+//            (BM x 64 elements, 16-byte chunks XOR-swizzled by row so that the
+//            operand reads are bank-conflict free), double buffered, one
+//            barrier per K-step.
+// Workgroup ids are mapped so that the eight XCDs (id mod 8) each take their
+// own column blocks and walk the slot blocks fastest: workgroups that run
+// together on an XCD share the expert's weight tile in that XCD's L2.
+#include "vec16.h"
+#include "launch.h"
+
+namespace sarathi_hip {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kGemmBN = 256;   // output columns per workgroup
+constexpr int kGemmBK = 64;    // K elements per pipeline step
+constexpr int kGemmWaveN = 64; // output columns per wave
+
+template <int DT> SK_DEV f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+  if constexpr (DT == kBF16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+struct MoeGemmArgs {
+  const void* a;            // [tokens, K]
+  const void* b;            // [E, N, K]
+  void* c;                  // [tokens * top_k, N]
+  const float* topk_weights;        // flat [tokens * top_k] or null
+  const int32_t* sorted_token_ids;  // [em]
+  const int32_t* expert_ids;        // [ceil(em / BM)]
+  const int32_t* num_tokens_post_padded;
+  int64_t a_row_stride;     // elements
+  int64_t b_expert_stride;  // elements
+  int64_t c_row_stride;     // elements
+  int32_t num_valid;        // tokens * top_k
+  int32_t em;               // length of sorted_token_ids
+  int32_t N, K;
+  int32_t top_k;
+  int32_t m_blocks, n_blocks;
+};
+
+template <int DT, int BM, bool MUL_WEIGHT>
+__global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmArgs g) {
+  constexpr int MT = BM / 32;          // token tiles per wave
+  constexpr int NT = kGemmWaveN / 32;  // weight tiles per wave
+  constexpr int SUB = kGemmBK / 16;    // MFMA sub-steps per K-step
+  constexpr int A_LOADS = BM / 32;     // 16-byte chunks each thread gathers per K-step
+  __shared__ u32x4 tok_lds[2][BM * 8];  // [buffer][row * 8 + swizzled chunk]
+
+  // ---- which tile
+  const unsigned id = blockIdx.x;
+  const unsigned xcd = id & 7u, t = id >> 3;
+  const int pid_m = t % g.m_blocks;
+  const int pid_n = (t / g.m_blocks) * 8 + xcd;
+  if (pid_n >= g.n_blocks) return;
+  if (pid_m * BM >= *g.num_tokens_post_padded) return;
+  const int expert = g.expert_ids[pid_m];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int l32 = lane & 31, grp = lane >> 5;
+
+  // ---- weights: buffer resource over the expert's [N, K] matrix; rows >= N read as zero
+  const int64_t b_bytes = (int64_t)g.N * g.K * 2;
+  const rsrc_t rb = make_rsrc(reinterpret_cast<const char*>(g.b) + (int64_t)expert * g.b_expert_stride * 2,
+                              (uint32_t)b_bytes);
+  const int n_wave0 = pid_n * kGemmBN + wave * kGemmWaveN;
+  uint32_t w_off[NT];  // byte offset of this lane's row at k = 0, chunk `grp`
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int n = n_wave0 + nt * 32 + l32;
+    w_off[nt] = n < g.N ? (uint32_t)n * (uint32_t)g.K * 2u + grp * 16u : 0x80000000u;
+  }
+
+  // ---- tokens: each thread gathers chunk `tid & 7` of rows (tid >> 3) + 32 j
+  const int a_chunk = tid & 7;
+  const char* a_ptr[A_LOADS];
+#pragma unroll
+  for (int j = 0; j < A_LOADS; ++j) {
+    const int r = (tid >> 3) + 32 * j;
+    const int slot_index = pid_m * BM + r;
+    const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
+    a_ptr[j] = sid < g.num_valid
+                   ? reinterpret_cast<const char*>(g.a) + ((int64_t)(sid / g.top_k) * g.a_row_stride) * 2 + a_chunk * 16
+                   : nullptr;
+  }
+  auto gather = [&](int k0, u32x4 (&regs)[A_LOADS]) {
+#pragma unroll
+    for (int j = 0; j < A_LOADS; ++j)
+      regs[j] = a_ptr[j] ? *reinterpret_cast<const u32x4*>(a_ptr[j] + (int64_t)k0 * 2)
+                         : (u32x4){0, 0, 0, 0};
+  };
+  auto stage = [&](int buf, const u32x4 (&regs)[A_LOADS]) {
+#pragma unroll
+    for (int j = 0; j < A_LOADS; ++j) {
+      const int r = (tid >> 3) + 32 * j;
+      tok_lds[buf][r * 8 + (a_chunk ^ (r & 7))] = regs[j];
+    }
+  };
+  auto load_weights = [&](int k0, u32x4 (&w)[NT][SUB]) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int s = 0; s < SUB; ++s)
+        w[nt][s] = buf_load16<kCached>(rb, w_off[nt] + (uint32_t)(k0 + s * 16) * 2u);
+  };
+
+  f32x16 acc[NT][MT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[nt][mt][i] = 0.f;
+
+  u32x4 wcur[NT][SUB], wnext[NT][SUB], anext[A_LOADS];
+  gather(0, anext);
+  load_weights(0, wcur);
+  stage(0, anext);
+  __syncthreads();
+
+  const int steps = g.K / kGemmBK;
+  for (int step = 0; step < steps; ++step) {
+    const int cur = step & 1;
+    const bool more = step + 1 < steps;
+    if (more) {
+      gather((step + 1) * kGemmBK, anext);
+      load_weights((step + 1) * kGemmBK, wnext);
+    }
+#pragma unroll
+    for (int s = 0; s < SUB; ++s) {
+      u32x4 tokv[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int r = mt * 32 + l32;
+        tokv[mt] = tok_lds[cur][r * 8 + ((2 * s + grp) ^ (r & 7))];
+      }
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = mfma32<DT>(wcur[nt][s], tokv[mt], acc[nt][mt]);
+    }
+    if (more) {
+      stage(cur ^ 1, anext);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int s = 0; s < SUB; ++s) wcur[nt][s] = wnext[nt][s];
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane holds, per accumulator quad, 4 consecutive columns of one token
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int slot_index = pid_m * BM + mt * 32 + l32;
+    const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
+    if (sid >= g.num_valid) continue;
+    float scale = 1.f;
+    if constexpr (MUL_WEIGHT) scale = g.topk_weights[sid];
+    char* crow = reinterpret_cast<char*>(g.c) + (int64_t)sid * g.c_row_stride * 2;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n_wave0 + nt * 32 + q * 8 + grp * 4;
+        float v0 = acc[nt][mt][q * 4 + 0], v1 = acc[nt][mt][q * 4 + 1];
+        float v2 = acc[nt][mt][q * 4 + 2], v3 = acc[nt][mt][q * 4 + 3];
+        if constexpr (MUL_WEIGHT) { v0 *= scale; v1 *= scale; v2 *= scale; v3 *= scale; }
+        if (n + 3 < g.N) {
+          u32x2 out = {pack2<DT>(v0, v1), pack2<DT>(v2, v3)};
+          *reinterpret_cast<u32x2*>(crow + (int64_t)n * 2) = out;
+        } else {
+          const float v[4] = {v0, v1, v2, v3};
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < g.N) store_elem<DT>(crow, n + e, v[e]);
+        }
+      }
+    }
+  }
+}
+
+template <int DT, int BM>
+static int launch_moe_gemm(const MoeGemmArgs& g, bool mul_weight, hipStream_t st) {
+  const int64_t groups = (g.n_blocks + 7) / 8;
+  const int64_t blocks = groups * g.m_blocks * 8;
+  if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
+  if (mul_weight)
+    hipLaunchKernelGGL((moe_gemm_kernel<DT, BM, true>), dim3((unsigned)blocks), dim3(256), 0, st, g);
+  else
+    hipLaunchKernelGGL((moe_gemm_kernel<DT, BM, false>), dim3((unsigned)blocks), dim3(256), 0, st, g);
+  return launch_status();
+}
+
+}  // namespace sarathi_hip
+
+extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
+                                        const float* topk_weights,
+                                        const int32_t* sorted_token_ids,
+                                        const int32_t* expert_ids,
+                                        const int32_t* num_tokens_post_padded,
+                                        int64_t num_valid_tokens, int64_t sorted_len, int64_t n,
+                                        int64_t k, int64_t a_row_stride, int64_t b_expert_stride,
+                                        int64_t c_row_stride, int block_m, int top_k,
+                                        int mul_routed_weight, int dtype, void* stream) {
+  using namespace sarathi_hip;
+  if (!a || !b || !c || !sorted_token_ids || !expert_ids || !num_tokens_post_padded)
+    return SARATHI_ERR_INVALID_ARG;
+  if (mul_routed_weight && !topk_weights) return SARATHI_ERR_INVALID_ARG;
+  if (num_valid_tokens < 0 || sorted_len < 0 || n <= 0 || k <= 0 || top_k <= 0 ||
+      a_row_stride < k || c_row_stride < n || b_expert_stride < n * k)
+    return SARATHI_ERR_INVALID_ARG;
+  if (block_m != 32 && block_m != 64 && block_m != 128) return SARATHI_ERR_UNSUPPORTED;
+  if (dtype != kBF16 && dtype != kF16) return SARATHI_ERR_UNSUPPORTED;
+  // 16-byte operand pieces and whole K-steps; one buffer resource per expert matrix
+  if (k % kGemmBK != 0 || a_row_stride % 8 != 0 || b_expert_stride % 8 != 0 || n % 4 != 0 ||
+      c_row_stride % 4 != 0 || !aligned16(a) || !aligned16(b) || (reinterpret_cast<uintptr_t>(c) & 7u))
+    return SARATHI_ERR_UNSUPPORTED;
+  if (n * k * 2 >= 0x80000000LL || num_valid_tokens > 0x7fffffffLL || sorted_len > 0x7fffffffLL)
+    return SARATHI_ERR_UNSUPPORTED;
+  if (sorted_len == 0 || num_valid_tokens == 0) return SARATHI_OK;
+  MoeGemmArgs g;
+  g.a = a; g.b = b; g.c = c;
+  g.topk_weights = topk_weights;
+  g.sorted_token_ids = sorted_token_ids;
+  g.expert_ids = expert_ids;
+  g.num_tokens_post_padded = num_tokens_post_padded;
+  g.a_row_stride = a_row_stride;
+  g.b_expert_stride = b_expert_stride;
+  g.c_row_stride = c_row_stride;
+  g.num_valid = (int32_t)num_valid_tokens;
+  g.em = (int32_t)sorted_len;
+  g.N = (int32_t)n; g.K = (int32_t)k;
+  g.top_k = top_k;
+  g.m_blocks = (int32_t)((sorted_len + block_m - 1) / block_m);
+  g.n_blocks = (int32_t)((n + kGemmBN - 1) / kGemmBN);
+  hipStream_t st = (hipStream_t)stream;
+  const bool mw = mul_routed_weight != 0;
+#define SK_GEMM(DT)                                                       \
+  switch (block_m) {                                                      \
+    case 32: return launch_moe_gemm<DT, 32>(g, mw, st);                   \
+    case 64: return launch_moe_gemm<DT, 64>(g, mw, st);                   \
+    default: return launch_moe_gemm<DT, 128>(g, mw, st);                  \
+  }
+  if (dtype == kBF16) { SK_GEMM(kBF16) } else { SK_GEMM(kF16) }
+#undef SK_GEMM
+}

@@ -280,6 +280,52 @@ void moe_align_block_size_filled(torch::Tensor topk_ids, int64_t num_experts, in
                  num_tokens_post_pad, true, "moe_align_block_size_filled");
 }
 
+// A [tokens, K], B [E, N, K], C [tokens, topk, N] (or any tensor whose rows of N elements are
+// addressed by slot = token * topk + j), as invoke_fused_moe_kernel passes them.
+void moe_grouped_gemm(torch::Tensor& a, torch::Tensor& b, torch::Tensor& c,
+                      torch::Tensor& topk_weights, torch::Tensor& sorted_token_ids,
+                      torch::Tensor& expert_ids, torch::Tensor& num_tokens_post_padded,
+                      int64_t num_valid_tokens, int64_t block_m, int64_t top_k,
+                      bool mul_routed_weight) {
+  const char* op = "moe_grouped_gemm";
+  check_gpu(a, a, op, "A");
+  check_gpu(b, a, op, "B");
+  check_gpu(c, a, op, "C");
+  check_gpu(topk_weights, a, op, "topk_weights");
+  check_gpu(sorted_token_ids, a, op, "sorted_token_ids");
+  check_gpu(expert_ids, a, op, "expert_ids");
+  check_gpu(num_tokens_post_padded, a, op, "num_tokens_post_padded");
+  TORCH_CHECK(a.dim() == 2 && b.dim() == 3 && a.size(1) == b.size(2), op,
+              ": A must be [tokens, K] and B [E, N, K]");
+  TORCH_CHECK(a.scalar_type() == b.scalar_type() && c.scalar_type() == a.scalar_type(), op,
+              ": A, B and C must share a dtype");
+  TORCH_CHECK(a.scalar_type() == at::ScalarType::BFloat16 || a.scalar_type() == at::ScalarType::Half,
+              op, ": only bfloat16 and float16 are supported");
+  TORCH_CHECK(a.stride(1) == 1 && b.stride(2) == 1 && b.stride(1) == b.size(2) && c.is_contiguous(),
+              op, ": A rows, B matrices and C must be contiguous");
+  TORCH_CHECK(c.size(-1) == b.size(1) && c.numel() == num_valid_tokens * b.size(1), op,
+              ": C must hold num_valid_tokens rows of N elements");
+  TORCH_CHECK(topk_weights.scalar_type() == at::ScalarType::Float && topk_weights.is_contiguous() &&
+                  topk_weights.numel() >= (mul_routed_weight ? num_valid_tokens : 0),
+              op, ": topk_weights must be contiguous float32 [tokens, topk]");
+  TORCH_CHECK(sorted_token_ids.scalar_type() == at::ScalarType::Int &&
+                  expert_ids.scalar_type() == at::ScalarType::Int &&
+                  num_tokens_post_padded.scalar_type() == at::ScalarType::Int &&
+                  sorted_token_ids.is_contiguous() && expert_ids.is_contiguous(),
+              op, ": routing tensors must be contiguous int32");
+  TORCH_CHECK(block_m > 0 && expert_ids.numel() * block_m >= sorted_token_ids.numel(), op,
+              ": expert_ids is too short for sorted_token_ids and block_m");
+  LaunchScope scope(a);
+  raise_on(sarathi_moe_grouped_gemm(
+               a.data_ptr(), b.data_ptr(), c.data_ptr(), topk_weights.data_ptr<float>(),
+               sorted_token_ids.data_ptr<int32_t>(), expert_ids.data_ptr<int32_t>(),
+               num_tokens_post_padded.data_ptr<int32_t>(), num_valid_tokens,
+               sorted_token_ids.numel(), b.size(1), b.size(2), a.stride(0), b.stride(0), b.size(1),
+               (int)block_m, (int)top_k, mul_routed_weight ? 1 : 0, dtype_code(a, op),
+               scope.stream),
+           op);
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -304,4 +350,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "stable sort of token ids by expert, runs padded to block_size");
   m.def("moe_align_block_size_filled", &moe_align_block_size_filled,
         "moe_align_block_size that also writes the padding value into unused slots");
+  m.def("moe_grouped_gemm", &moe_grouped_gemm,
+        "C[slot] = A[slot / top_k] @ B[expert(slot)]^T over moe_align_block_size's layout");
 }

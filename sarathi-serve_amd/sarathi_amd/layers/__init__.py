@@ -3,6 +3,7 @@
 layers/fused_moe/fused_moe.py).  Same class / function names and call signatures, so model code written
 against the reference's layers runs unchanged; the bodies call this package's HIP ops."""
 from .activation import FastGELU, NewGELU, SiluAndMul, get_act_fn
+from .fused_moe import fused_experts, fused_moe, invoke_fused_moe_kernel
 from .moe_routing import fused_topk, moe_align_block_size
 from .norm import RMSNorm
 from .rotary import (DynamicNTKScalingRotaryEmbedding, LinearScalingRotaryEmbedding,
@@ -10,4 +11,5 @@ from .rotary import (DynamicNTKScalingRotaryEmbedding, LinearScalingRotaryEmbedd
 
 __all__ = ["RMSNorm", "SiluAndMul", "NewGELU", "FastGELU", "get_act_fn", "RotaryEmbedding",
            "LinearScalingRotaryEmbedding", "DynamicNTKScalingRotaryEmbedding",
-           "YaRNScalingRotaryEmbedding", "get_rope", "fused_topk", "moe_align_block_size"]
+           "YaRNScalingRotaryEmbedding", "get_rope", "fused_topk", "moe_align_block_size",
+           "invoke_fused_moe_kernel", "fused_experts", "fused_moe"]

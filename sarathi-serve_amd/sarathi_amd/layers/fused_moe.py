@@ -1,0 +1,104 @@
+"""Fused MoE forward on this package's ops (reference:
+sarathi/model_executor/layers/fused_moe/fused_moe.py:207-260 and :411-622).
+
+``fused_moe`` = top-k routing -> slot sort (moe_align_block_size) -> grouped GEMM with w1 ->
+silu_and_mul -> grouped GEMM with w2 (times the routing weight) -> sum over the k slots of a token.
+The two GEMMs are one hand-written MFMA kernel (csrc/moe_gemm.hip) instead of the reference's
+Triton kernel; there are no tuning JSON files, the slot-block size is picked from the batch size.
+fp8 weights / scales are not supported.
+"""
+from typing import Any, Dict, Optional
+
+import torch
+
+from .. import activation_ops, moe_ops
+from .moe_routing import fused_topk, moe_align_block_size
+
+_BLOCK_SIZES = (32, 64, 128)
+CHUNK_SIZE = 64 * 1024     # tokens per pass, as in the reference (fused_moe.py:459)
+
+
+def get_default_config(M: int, E: int, N: int, K: int, topk: int,
+                       dtype: Optional[str] = None) -> Dict[str, int]:
+    """Slot-block size for M tokens: the more slots an expert receives, the taller the tile (a
+    taller tile re-uses each weight fragment for more tokens).  BLOCK_SIZE_N / BLOCK_SIZE_K are
+    fixed properties of the kernel and reported for information."""
+    per_expert = M * topk / max(E, 1)
+    block_m = 128 if per_expert >= 512 else 64 if per_expert >= 96 else 32
+    return {"BLOCK_SIZE_M": block_m, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 64, "GROUP_SIZE_M": 1}
+
+
+def invoke_fused_moe_kernel(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor,
+                            A_scale: Optional[torch.Tensor], B_scale: Optional[torch.Tensor],
+                            topk_weights: torch.Tensor, topk_ids: torch.Tensor,
+                            sorted_token_ids: torch.Tensor, expert_ids: torch.Tensor,
+                            num_tokens_post_padded: torch.Tensor, mul_routed_weight: bool,
+                            top_k: int, config: Dict[str, Any], compute_type=None) -> None:
+    """Same argument list as the reference's launcher.  ``config["BLOCK_SIZE_M"]`` must be the block
+    size ``sorted_token_ids`` was aligned with."""
+    assert A_scale is None and B_scale is None, "fp8 scales are not supported"
+    assert topk_weights.stride(1) == 1 and sorted_token_ids.stride(0) == 1
+    block_m = int(config["BLOCK_SIZE_M"])
+    if block_m not in _BLOCK_SIZES:
+        raise ValueError(f"BLOCK_SIZE_M must be one of {_BLOCK_SIZES}, got {block_m}")
+    moe_ops.moe_grouped_gemm(A, B, C, topk_weights, sorted_token_ids, expert_ids,
+                             num_tokens_post_padded, topk_ids.numel(), block_m, top_k,
+                             bool(mul_routed_weight))
+
+
+def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
+                  topk_weights: torch.Tensor, topk_ids: torch.Tensor, inplace: bool = False,
+                  override_config: Optional[Dict[str, Any]] = None,
+                  w1_scale: Optional[torch.Tensor] = None, w2_scale: Optional[torch.Tensor] = None,
+                  a1_scale: Optional[torch.Tensor] = None,
+                  a2_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    assert hidden_states.shape[1] == w1.shape[2], "Hidden size mismatch"
+    assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
+    assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
+    assert w1.is_contiguous() and w2.is_contiguous(), "Expert weights must be contiguous"
+    assert hidden_states.dtype in (torch.float16, torch.bfloat16)
+    assert w1_scale is None and w2_scale is None and a1_scale is None and a2_scale is None, \
+        "fp8 scales are not supported"
+    num_tokens, K = hidden_states.shape
+    E, N, _ = w1.shape
+    topk = topk_ids.shape[1]
+    dev, dt = hidden_states.device, hidden_states.dtype
+    M = min(num_tokens, CHUNK_SIZE)
+    cache1 = torch.empty((M, topk, N), device=dev, dtype=dt)
+    cache2 = torch.empty((M * topk, N // 2), device=dev, dtype=dt)
+    cache3 = torch.empty((M, topk, w2.shape[1]), device=dev, dtype=dt)
+    out = hidden_states if inplace else torch.empty_like(hidden_states)
+    topk_weights = topk_weights.contiguous()
+    for begin in range(0, num_tokens, CHUNK_SIZE):
+        end = min(begin + CHUNK_SIZE, num_tokens)
+        n = end - begin
+        cur_hidden = hidden_states[begin:end]
+        cur_ids, cur_w = topk_ids[begin:end], topk_weights[begin:end]
+        config = override_config or get_default_config(n, E, w2.shape[1], K, topk)
+        c1, c2, c3 = cache1[:n], cache2[:n * topk], cache3[:n]
+        sorted_ids, expert_ids, post_padded = moe_align_block_size(cur_ids, config["BLOCK_SIZE_M"], E)
+        invoke_fused_moe_kernel(cur_hidden, w1, c1, None, None, cur_w, cur_ids, sorted_ids,
+                                expert_ids, post_padded, False, topk, config)
+        activation_ops.silu_and_mul(c2, c1.view(-1, N))
+        invoke_fused_moe_kernel(c2, w2, c3, None, None, cur_w, cur_ids, sorted_ids, expert_ids,
+                                post_padded, True, 1, config)
+        torch.sum(c3, dim=1, out=out[begin:end])
+    return out
+
+
+def fused_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
+              gating_output: torch.Tensor, topk: int, renormalize: bool, inplace: bool = False,
+              override_config: Optional[Dict[str, Any]] = None, use_grouped_topk: bool = False,
+              num_expert_group: Optional[int] = None, topk_group: Optional[int] = None,
+              w1_scale: Optional[torch.Tensor] = None, w2_scale: Optional[torch.Tensor] = None,
+              a1_scale: Optional[torch.Tensor] = None,
+              a2_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """MoE layer forward: ``hidden_states [T, H]``, ``w1 [E, 2I, H]``, ``w2 [E, H, I]``,
+    ``gating_output [T, E]`` (logits)."""
+    assert gating_output.shape[1] == w1.shape[0], "Number of experts mismatch"
+    if use_grouped_topk:
+        raise NotImplementedError("grouped_topk (DeepSeek-V2 routing) is not part of this library")
+    topk_weights, topk_ids = fused_topk(hidden_states, gating_output, topk, renormalize)
+    return fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, inplace=inplace,
+                         override_config=override_config, w1_scale=w1_scale, w2_scale=w2_scale,
+                         a1_scale=a1_scale, a2_scale=a2_scale)

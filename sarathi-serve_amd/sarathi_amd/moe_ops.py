@@ -11,6 +11,9 @@ topk_softmax = _C.topk_softmax
 moe_align_block_size = _C.moe_align_block_size
 topk_softmax_renorm = _C.topk_softmax_renorm
 moe_align_block_size_filled = _C.moe_align_block_size_filled
+# grouped expert GEMM over moe_align_block_size's layout: what the reference launches as a Triton
+# kernel from invoke_fused_moe_kernel (layers/fused_moe/fused_moe.py:207-260)
+moe_grouped_gemm = _C.moe_grouped_gemm
 
 __all__ = ["topk_softmax", "moe_align_block_size", "topk_softmax_renorm",
-           "moe_align_block_size_filled"]
+           "moe_align_block_size_filled", "moe_grouped_gemm"]

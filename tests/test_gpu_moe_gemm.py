@@ -1,0 +1,109 @@
+"""GPU: the grouped expert GEMM (the consumer of moe_align_block_size's layout) and the whole
+fused MoE forward, against CPU formulations in fp32.
+
+The contraction's accumulation order is not defined by the reference (Triton's tl.dot), so the
+comparison is by tolerance: |got - want| <= 1e-2 * max|want| + 1e-2 * |want| for bf16/fp16
+outputs.  The identity-weight case has exactly one non-zero product per output and must be exact.
+"""
+import pytest
+import torch
+
+from helpers import gen, randn
+from oracle import c_oracle, torch_formulations
+
+pytestmark = pytest.mark.gpu
+
+
+def _route(T, E, k, B, seed):
+    g = gen(seed)
+    gating = torch.randn((T, E), generator=g, dtype=torch.float32)
+    w = torch.empty((T, k))
+    ids = torch.empty((T, k), dtype=torch.int32)
+    src = torch.empty((T, k), dtype=torch.int32)
+    c_oracle.topk_softmax(w, ids, src, gating)
+    n = T * k + E * (B - 1)
+    s = torch.full((n,), T * k, dtype=torch.int32)
+    e = torch.zeros(((n + B - 1) // B,), dtype=torch.int32)
+    p = torch.zeros((1,), dtype=torch.int32)
+    c_oracle.moe_align_block_size(ids, E, B, s, e, p)
+    return gating, w, ids, s, e, p
+
+
+def _close(got, want, what):
+    got, want = got.float().cpu(), want.float()
+    tol = 1e-2 * want.abs().max().item() + 1e-2 * want.abs()
+    bad = (got - want).abs() > tol
+    assert not bool(bad.any()), "%s: %d elements outside tolerance, max diff %.4g" % (
+        what, int(bad.sum()), (got - want).abs().max().item())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,k,BM,N,K,mul", [
+    (300, 8, 2, 64, 512, 256, False),
+    (300, 8, 2, 64, 512, 256, True),
+    (77, 4, 2, 32, 260, 128, True),      # N not a multiple of the 256-wide tile nor of 32
+    (1000, 8, 2, 128, 768, 512, False),
+    (33, 16, 4, 32, 256, 64, True),      # some experts empty, single K step
+    (5, 8, 1, 32, 1024, 192, False),
+])
+def test_grouped_gemm_matches_formulation(ops, dev, dtype, T, E, k, BM, N, K, mul):
+    _, w, ids, s, e, p = _route(T, E, k, BM, T + N)
+    g = gen(K)
+    A = randn((T, K), g, dtype, std=0.5)
+    Bw = randn((E, N, K), g, dtype, std=0.5)
+    want = torch.zeros((T, k, N), dtype=dtype)
+    torch_formulations.moe_grouped_gemm(A, Bw, want, w, s, e, p, T * k, BM, k, mul)
+    got = torch.full((T, k, N), 7.0, dtype=dtype, device=dev)
+    ops.moe_ops.moe_grouped_gemm(A.to(dev), Bw.to(dev), got, w.to(dev), s.to(dev), e.to(dev),
+                                 p.to(dev), T * k, BM, k, mul)
+    _close(got, want, "grouped gemm")
+
+
+def test_grouped_gemm_second_stage_addressing(ops, dev):
+    """top_k = 1 addressing of the down projection: A rows are slots (tokens * topk of them)."""
+    T, E, k, BM, N, K = 200, 8, 2, 64, 256, 128
+    _, w, ids, s, e, p = _route(T, E, k, BM, 5)
+    g = gen(6)
+    A = randn((T * k, K), g, std=0.5)
+    Bw = randn((E, N, K), g, std=0.5)
+    want = torch.zeros((T, k, N), dtype=torch.bfloat16)
+    torch_formulations.moe_grouped_gemm(A, Bw, want, w, s, e, p, T * k, BM, 1, True)
+    got = torch.zeros((T, k, N), dtype=torch.bfloat16, device=dev)
+    ops.moe_ops.moe_grouped_gemm(A.to(dev), Bw.to(dev), got, w.to(dev), s.to(dev), e.to(dev),
+                                 p.to(dev), T * k, BM, 1, True)
+    _close(got, want, "second stage")
+
+
+def test_grouped_gemm_identity_weights_exact(ops, dev):
+    """B[e] = 2^e * I: every output has a single non-zero product, so C[slot] = 2^e * A[token]
+    exactly; this pins operand layout, expert selection and slot addressing bit for bit."""
+    T, E, k, BM, K = 500, 8, 2, 64, 256
+    _, w, ids, s, e, p = _route(T, E, k, BM, 9)
+    g = gen(10)
+    A = randn((T, K), g)
+    Bw = torch.stack([torch.eye(K) * (2.0 ** x) for x in range(E)]).bfloat16()
+    got = torch.zeros((T, k, K), dtype=torch.bfloat16, device=dev)
+    ops.moe_ops.moe_grouped_gemm(A.to(dev), Bw.to(dev), got, w.to(dev), s.to(dev), e.to(dev),
+                                 p.to(dev), T * k, BM, k, False)
+    want = A.float().unsqueeze(1) * torch.pow(2.0, ids.float()).unsqueeze(-1)
+    assert torch.equal(got.float().cpu(), want)
+
+
+@pytest.mark.parametrize("T,E,k,H,I,renorm", [(64, 8, 2, 256, 512, True), (700, 8, 2, 512, 1024, True),
+                                            (129, 4, 1, 256, 256, False)])
+def test_fused_moe_forward(ops, dev, T, E, k, H, I, renorm):
+    from sarathi_amd import layers
+    g = gen(T)
+    x = randn((T, H), g, std=1.0)
+    w1 = randn((E, 2 * I, H), g, std=H ** -0.5)
+    w2 = randn((E, H, I), g, std=I ** -0.5)
+    gating = torch.randn((T, E), generator=g, dtype=torch.float32)
+    want = torch_formulations.fused_moe(x, w1, w2, gating, k, renorm)
+    got = layers.fused_moe(x.to(dev), w1.to(dev), w2.to(dev), gating.to(dev), k, renorm)
+    assert got.shape == (T, H) and got.dtype == torch.bfloat16
+    _close(got, want, "fused_moe")
+    # in place
+    xd = x.to(dev)
+    out = layers.fused_moe(xd, w1.to(dev), w2.to(dev), gating.to(dev), k, renorm, inplace=True)
+    assert out.data_ptr() == xd.data_ptr()
+    _close(xd, want, "fused_moe inplace")
