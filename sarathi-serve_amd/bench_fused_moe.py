@@ -63,25 +63,38 @@ def main():
         torch.cuda.synchronize()
         return a.elapsed_time(b) / args.iters
 
-    g1 = lambda: ops.moe_ops.moe_grouped_gemm(x, w1, c1, tw, s, e, p, T * k, bm, k, False)  # noqa: E731
-    g2 = lambda: ops.moe_ops.moe_grouped_gemm(c2, w2, c3, tw, s, e, p, T * k, bm, 1, True)  # noqa: E731
-    ms1 = timeit(g1)
-    ops.activation_ops.silu_and_mul(c2, c1.view(-1, 2 * I))
-    ms2 = timeit(g2)
-    ms_all = timeit(lambda: layers.fused_moe(x, w1, w2, gating, k, True, override_config=config))
     f1 = 2.0 * T * k * H * 2 * I
     f2 = 2.0 * T * k * I * H
+    res = {}
+    for label in ("row_major", "packed"):
+        if label == "packed":      # re-tile once, then drop the row-major copies
+            p1, p2 = layers.pack_expert_weights(w1), layers.pack_expert_weights(w2)
+            b1, b2, pk = p1.data, p2.data, True
+            del w1, w2
+            torch.cuda.empty_cache()
+            wa, wb = p1, p2
+        else:
+            b1, b2, pk, wa, wb = w1, w2, False, w1, w2
+        g1 = lambda: ops.moe_ops.moe_grouped_gemm(x, b1, c1, tw, s, e, p, T * k, bm, k, False, pk, 2 * I)  # noqa: E731
+        g2 = lambda: ops.moe_ops.moe_grouped_gemm(c2, b2, c3, tw, s, e, p, T * k, bm, 1, True, pk, H)  # noqa: E731
+        ms1 = timeit(g1)
+        ops.activation_ops.silu_and_mul(c2, c1.view(-1, 2 * I))
+        ms2 = timeit(g2)
+        ms_all = timeit(lambda: layers.fused_moe(x, wa, wb, gating, k, True, override_config=config))
+        res[label] = {
+            "gemm_w1": {"ms": round(ms1, 4), "TFLOPs": round(f1 / ms1 * 1e-9, 1),
+                        "frac_of_mfma_peak": round(f1 / ms1 * 1e-9 / MFMA_PEAK_TFLOPS, 4)},
+            "gemm_w2": {"ms": round(ms2, 4), "TFLOPs": round(f2 / ms2 * 1e-9, 1),
+                        "frac_of_mfma_peak": round(f2 / ms2 * 1e-9 / MFMA_PEAK_TFLOPS, 4)},
+            "fused_moe_forward": {"ms": round(ms_all, 4),
+                                  "TFLOPs": round((f1 + f2) / ms_all * 1e-9, 1)},
+        }
     out = {
         "metric": "grouped expert GEMM TFLOP/s (Mixtral-8x7B MoE layer shape)",
         "config": {"tokens": T, "experts": E, "topk": k, "hidden": H, "intermediate": I,
                    "dtype": "bf16", "block_m": bm, "device": torch.cuda.get_device_name(0)},
-        "gemm_w1": {"ms": round(ms1, 4), "TFLOPs": round(f1 / ms1 * 1e-9, 1),
-                    "frac_of_mfma_peak": round(f1 / ms1 * 1e-9 / MFMA_PEAK_TFLOPS, 4)},
-        "gemm_w2": {"ms": round(ms2, 4), "TFLOPs": round(f2 / ms2 * 1e-9, 1),
-                    "frac_of_mfma_peak": round(f2 / ms2 * 1e-9 / MFMA_PEAK_TFLOPS, 4)},
-        "fused_moe_forward": {"ms": round(ms_all, 4),
-                              "TFLOPs": round((f1 + f2) / ms_all * 1e-9, 1)},
-        "weight_bytes": (w1.numel() + w2.numel()) * 2,
+        "weights": res,
+        "weight_bytes": (E * 2 * I * H + E * H * I) * 2,
     }
     print(json.dumps(out))
 

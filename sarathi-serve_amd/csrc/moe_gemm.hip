@@ -17,7 +17,16 @@
 // epilogue writes 8-byte pieces of C rows.
 //   weights  never shared between waves: each lane loads its 16-byte operand
 //            pieces straight from global memory (buffer loads on the expert's
-//            matrix, clipped at N rows), one K-step (64) ahead of their use;
+//            matrix, clipped at N rows) into the register slot that the MFMAs of
+//            the current K-step have just consumed, i.e. one K-step (64) ahead
+//            of their use, with no second register buffer.  Two layouts of B:
+//              row-major [E, N, K] (the reference's): a wave's operand load
+//                touches 32 rows x 32 bytes, which makes the texture-address
+//                unit, not the MFMA pipe, the limit (~22-36 % of peak);
+//              packed    [E, N/32, K/16, 64 lanes, 8]: the 1 KiB a wave needs for
+//                one 32x16 operand is contiguous in lane order, one fully
+//                coalesced load (~1.3-1.9x faster).  Weights are static, so
+//                packing them once at load time is free.
 //   tokens   shared by the four waves: gathered once per K-step into LDS
 //            (BM x 64 elements, 16-byte chunks XOR-swizzled by row so that the
 //            operand reads are bank-conflict free), double buffered, one
@@ -65,7 +74,7 @@ struct MoeGemmArgs {
   int32_t m_blocks, n_blocks;
 };
 
-template <int DT, int BM, bool MUL_WEIGHT>
+template <int DT, int BM, bool MUL_WEIGHT, bool PACKED>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmArgs g) {
   constexpr int MT = BM / 32;          // token tiles per wave
   constexpr int NT = kGemmWaveN / 32;  // weight tiles per wave
@@ -85,17 +94,28 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmArgs g) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int l32 = lane & 31, grp = lane >> 5;
 
-  // ---- weights: buffer resource over the expert's [N, K] matrix; rows >= N read as zero
-  const int64_t b_bytes = (int64_t)g.N * g.K * 2;
+  // ---- weights: buffer resource over the expert's matrix; rows >= N read as zero
+  const int n_wave0 = pid_n * kGemmBN + wave * kGemmWaveN;
+  const int n_tiles = (g.N + 31) >> 5;
+  const int64_t b_bytes = PACKED ? (int64_t)n_tiles * 32 * g.K * 2 : (int64_t)g.N * g.K * 2;
   const rsrc_t rb = make_rsrc(reinterpret_cast<const char*>(g.b) + (int64_t)expert * g.b_expert_stride * 2,
                               (uint32_t)b_bytes);
-  const int n_wave0 = pid_n * kGemmBN + wave * kGemmWaveN;
-  uint32_t w_off[NT];  // byte offset of this lane's row at k = 0, chunk `grp`
+  uint32_t w_off[NT];  // byte offset of this lane's operand piece at k = 0
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
-    const int n = n_wave0 + nt * 32 + l32;
-    w_off[nt] = n < g.N ? (uint32_t)n * (uint32_t)g.K * 2u + grp * 16u : 0x80000000u;
+    if constexpr (PACKED) {
+      const int tile = (n_wave0 >> 5) + nt;  // 32-row tile; its K/16 operand blocks of 1 KiB follow each other
+      w_off[nt] = tile < n_tiles ? (uint32_t)tile * (uint32_t)g.K * 64u + lane * 16u : 0x80000000u;
+    } else {
+      const int n = n_wave0 + nt * 32 + l32;
+      w_off[nt] = n < g.N ? (uint32_t)n * (uint32_t)g.K * 2u + grp * 16u : 0x80000000u;
+    }
   }
+  // operand piece of sub-step s (16 deep) of the K-step starting at k0
+  auto load_weight = [&](int nt, int k0, int s) {
+    return PACKED ? buf_load16<kCached>(rb, w_off[nt] + (uint32_t)((k0 >> 4) + s) * 1024u)
+                  : buf_load16<kCached>(rb, w_off[nt] + (uint32_t)(k0 + s * 16) * 2u);
+  };
 
   // ---- tokens: each thread gathers chunk `tid & 7` of rows (tid >> 3) + 32 j
   const int a_chunk = tid & 7;
@@ -122,14 +142,6 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmArgs g) {
       tok_lds[buf][r * 8 + (a_chunk ^ (r & 7))] = regs[j];
     }
   };
-  auto load_weights = [&](int k0, u32x4 (&w)[NT][SUB]) {
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-      for (int s = 0; s < SUB; ++s)
-        w[nt][s] = buf_load16<kCached>(rb, w_off[nt] + (uint32_t)(k0 + s * 16) * 2u);
-  };
-
   f32x16 acc[NT][MT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
@@ -138,40 +150,56 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmArgs g) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[nt][mt][i] = 0.f;
 
-  u32x4 wcur[NT][SUB], wnext[NT][SUB], anext[A_LOADS];
-  gather(0, anext);
-  load_weights(0, wcur);
+  // Note: the workgroups that share a weight tile (the slot blocks of one expert, side by side
+  // on one XCD) deliberately walk K in lockstep from 0.  Rotating their starting offsets was
+  // measured and is ~1.8x slower: the tile then has to stay in the 4 MB L2 for the whole loop
+  // instead of for one step.
+  const int steps = g.K / kGemmBK;
+  int kstep = 0;
+  u32x4 w[NT][SUB], anext[A_LOADS];
+  gather(kstep * kGemmBK, anext);
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int s = 0; s < SUB; ++s) w[nt][s] = load_weight(nt, kstep * kGemmBK, s);
   stage(0, anext);
   __syncthreads();
 
-  const int steps = g.K / kGemmBK;
+  // The loop body is branch-free so that the scheduler can keep loads, LDS reads and MFMAs
+  // interleaved: the last step simply loads the wrapped-around "next" K-step again (issued,
+  // never used), and the token operands of sub-step s + 1 are read from LDS before the MFMAs
+  // of sub-step s are issued.
+  auto read_tokens = [&](int buf, int s, u32x4 (&tokv)[MT]) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int r = mt * 32 + l32;
+      tokv[mt] = tok_lds[buf][r * 8 + ((2 * s + grp) ^ (r & 7))];
+    }
+  };
   for (int step = 0; step < steps; ++step) {
     const int cur = step & 1;
-    const bool more = step + 1 < steps;
-    if (more) {
-      gather((step + 1) * kGemmBK, anext);
-      load_weights((step + 1) * kGemmBK, wnext);
-    }
+    kstep = kstep + 1 < steps ? kstep + 1 : 0;
+    const int k_next = kstep * kGemmBK;
+    gather(k_next, anext);
+    u32x4 tokv[2][MT];
+    read_tokens(cur, 0, tokv[0]);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int s = 0; s < SUB; ++s) {
-      u32x4 tokv[MT];
+      if (s + 1 < SUB) read_tokens(cur, s + 1, tokv[(s + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);  // LDS reads of s + 1 are in flight under the MFMAs of s
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const int r = mt * 32 + l32;
-        tokv[mt] = tok_lds[cur][r * 8 + ((2 * s + grp) ^ (r & 7))];
+      for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[nt][mt] = mfma32<DT>(w[nt][s], tokv[s & 1][mt], acc[nt][mt]);
+        w[nt][s] = load_weight(nt, k_next, s);  // the slot is free again: refill it
       }
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = mfma32<DT>(wcur[nt][s], tokv[mt], acc[nt][mt]);
+      // keep this sub-step's loads here (a full K-step ahead of their use) and the LDS reads
+      // of the next sub-step ahead of its MFMAs
+      __builtin_amdgcn_sched_barrier(0);
     }
-    if (more) {
-      stage(cur ^ 1, anext);
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int s = 0; s < SUB; ++s) wcur[nt][s] = wnext[nt][s];
-    }
+    stage(cur ^ 1, anext);
     __syncthreads();
   }
 
@@ -207,14 +235,16 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmArgs g) {
 }
 
 template <int DT, int BM>
-static int launch_moe_gemm(const MoeGemmArgs& g, bool mul_weight, hipStream_t st) {
+static int launch_moe_gemm(const MoeGemmArgs& g, bool mul_weight, bool packed, hipStream_t st) {
   const int64_t groups = (g.n_blocks + 7) / 8;
   const int64_t blocks = groups * g.m_blocks * 8;
   if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
-  if (mul_weight)
-    hipLaunchKernelGGL((moe_gemm_kernel<DT, BM, true>), dim3((unsigned)blocks), dim3(256), 0, st, g);
-  else
-    hipLaunchKernelGGL((moe_gemm_kernel<DT, BM, false>), dim3((unsigned)blocks), dim3(256), 0, st, g);
+  const dim3 grid((unsigned)blocks), block(256);
+#define SK_LAUNCH(MW, PK) \
+  hipLaunchKernelGGL((moe_gemm_kernel<DT, BM, MW, PK>), grid, block, 0, st, g)
+  if (mul_weight) { if (packed) SK_LAUNCH(true, true); else SK_LAUNCH(true, false); }
+  else { if (packed) SK_LAUNCH(false, true); else SK_LAUNCH(false, false); }
+#undef SK_LAUNCH
   return launch_status();
 }
 
@@ -228,21 +258,25 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
                                         int64_t num_valid_tokens, int64_t sorted_len, int64_t n,
                                         int64_t k, int64_t a_row_stride, int64_t b_expert_stride,
                                         int64_t c_row_stride, int block_m, int top_k,
-                                        int mul_routed_weight, int dtype, void* stream) {
+                                        int mul_routed_weight, int b_layout, int dtype,
+                                        void* stream) {
   using namespace sarathi_hip;
   if (!a || !b || !c || !sorted_token_ids || !expert_ids || !num_tokens_post_padded)
     return SARATHI_ERR_INVALID_ARG;
   if (mul_routed_weight && !topk_weights) return SARATHI_ERR_INVALID_ARG;
   if (num_valid_tokens < 0 || sorted_len < 0 || n <= 0 || k <= 0 || top_k <= 0 ||
-      a_row_stride < k || c_row_stride < n || b_expert_stride < n * k)
+      a_row_stride < k || c_row_stride < n || b_expert_stride < n * k ||
+      (b_layout != SARATHI_MOE_B_ROW_MAJOR && b_layout != SARATHI_MOE_B_PACKED))
     return SARATHI_ERR_INVALID_ARG;
+  const bool packed = b_layout == SARATHI_MOE_B_PACKED;
+  if (packed && b_expert_stride < (n + 31) / 32 * 32 * k) return SARATHI_ERR_INVALID_ARG;
   if (block_m != 32 && block_m != 64 && block_m != 128) return SARATHI_ERR_UNSUPPORTED;
   if (dtype != kBF16 && dtype != kF16) return SARATHI_ERR_UNSUPPORTED;
   // 16-byte operand pieces and whole K-steps; one buffer resource per expert matrix
   if (k % kGemmBK != 0 || a_row_stride % 8 != 0 || b_expert_stride % 8 != 0 || n % 4 != 0 ||
       c_row_stride % 4 != 0 || !aligned16(a) || !aligned16(b) || (reinterpret_cast<uintptr_t>(c) & 7u))
     return SARATHI_ERR_UNSUPPORTED;
-  if (n * k * 2 >= 0x80000000LL || num_valid_tokens > 0x7fffffffLL || sorted_len > 0x7fffffffLL)
+  if ((n + 31) / 32 * 32 * k * 2 >= 0x80000000LL || num_valid_tokens > 0x7fffffffLL || sorted_len > 0x7fffffffLL)
     return SARATHI_ERR_UNSUPPORTED;
   if (sorted_len == 0 || num_valid_tokens == 0) return SARATHI_OK;
   MoeGemmArgs g;
@@ -264,9 +298,9 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
   const bool mw = mul_routed_weight != 0;
 #define SK_GEMM(DT)                                                       \
   switch (block_m) {                                                      \
-    case 32: return launch_moe_gemm<DT, 32>(g, mw, st);                   \
-    case 64: return launch_moe_gemm<DT, 64>(g, mw, st);                   \
-    default: return launch_moe_gemm<DT, 128>(g, mw, st);                  \
+    case 32: return launch_moe_gemm<DT, 32>(g, mw, packed, st);           \
+    case 64: return launch_moe_gemm<DT, 64>(g, mw, packed, st);           \
+    default: return launch_moe_gemm<DT, 128>(g, mw, packed, st);          \
   }
   if (dtype == kBF16) { SK_GEMM(kBF16) } else { SK_GEMM(kF16) }
 #undef SK_GEMM

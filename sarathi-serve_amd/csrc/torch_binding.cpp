@@ -281,12 +281,14 @@ void moe_align_block_size_filled(torch::Tensor topk_ids, int64_t num_experts, in
 }
 
 // A [tokens, K], B [E, N, K], C [tokens, topk, N] (or any tensor whose rows of N elements are
-// addressed by slot = token * topk + j), as invoke_fused_moe_kernel passes them.
+// addressed by slot = token * topk + j), as invoke_fused_moe_kernel passes them.  With
+// b_packed, B is the re-tiled weight tensor [E, ceil(N/32), K/16, 2, 32, 8] and `n` its logical
+// row count.
 void moe_grouped_gemm(torch::Tensor& a, torch::Tensor& b, torch::Tensor& c,
                       torch::Tensor& topk_weights, torch::Tensor& sorted_token_ids,
                       torch::Tensor& expert_ids, torch::Tensor& num_tokens_post_padded,
                       int64_t num_valid_tokens, int64_t block_m, int64_t top_k,
-                      bool mul_routed_weight) {
+                      bool mul_routed_weight, bool b_packed, int64_t n) {
   const char* op = "moe_grouped_gemm";
   check_gpu(a, a, op, "A");
   check_gpu(b, a, op, "B");
@@ -295,16 +297,26 @@ void moe_grouped_gemm(torch::Tensor& a, torch::Tensor& b, torch::Tensor& c,
   check_gpu(sorted_token_ids, a, op, "sorted_token_ids");
   check_gpu(expert_ids, a, op, "expert_ids");
   check_gpu(num_tokens_post_padded, a, op, "num_tokens_post_padded");
-  TORCH_CHECK(a.dim() == 2 && b.dim() == 3 && a.size(1) == b.size(2), op,
-              ": A must be [tokens, K] and B [E, N, K]");
+  TORCH_CHECK(a.dim() == 2 && a.stride(1) == 1, op, ": A must be [tokens, K] with contiguous rows");
+  const int64_t k = a.size(1);
+  int64_t expert_stride;
+  if (b_packed) {
+    TORCH_CHECK(b.dim() == 6 && b.is_contiguous() && b.size(3) == 2 && b.size(4) == 32 &&
+                    b.size(5) == 8 && b.size(2) * 16 == k && n > 0 && b.size(1) == (n + 31) / 32,
+                op, ": packed B must be contiguous [E, ceil(N/32), K/16, 2, 32, 8]");
+    expert_stride = b.stride(0);
+  } else {
+    TORCH_CHECK(b.dim() == 3 && b.size(2) == k && b.stride(2) == 1 && b.stride(1) == k, op,
+                ": B must be [E, N, K] with contiguous matrices");
+    n = b.size(1);
+    expert_stride = b.stride(0);
+  }
   TORCH_CHECK(a.scalar_type() == b.scalar_type() && c.scalar_type() == a.scalar_type(), op,
               ": A, B and C must share a dtype");
   TORCH_CHECK(a.scalar_type() == at::ScalarType::BFloat16 || a.scalar_type() == at::ScalarType::Half,
               op, ": only bfloat16 and float16 are supported");
-  TORCH_CHECK(a.stride(1) == 1 && b.stride(2) == 1 && b.stride(1) == b.size(2) && c.is_contiguous(),
-              op, ": A rows, B matrices and C must be contiguous");
-  TORCH_CHECK(c.size(-1) == b.size(1) && c.numel() == num_valid_tokens * b.size(1), op,
-              ": C must hold num_valid_tokens rows of N elements");
+  TORCH_CHECK(c.is_contiguous() && c.size(-1) == n && c.numel() == num_valid_tokens * n, op,
+              ": C must be contiguous and hold num_valid_tokens rows of N elements");
   TORCH_CHECK(topk_weights.scalar_type() == at::ScalarType::Float && topk_weights.is_contiguous() &&
                   topk_weights.numel() >= (mul_routed_weight ? num_valid_tokens : 0),
               op, ": topk_weights must be contiguous float32 [tokens, topk]");
@@ -320,8 +332,9 @@ void moe_grouped_gemm(torch::Tensor& a, torch::Tensor& b, torch::Tensor& c,
                a.data_ptr(), b.data_ptr(), c.data_ptr(), topk_weights.data_ptr<float>(),
                sorted_token_ids.data_ptr<int32_t>(), expert_ids.data_ptr<int32_t>(),
                num_tokens_post_padded.data_ptr<int32_t>(), num_valid_tokens,
-               sorted_token_ids.numel(), b.size(1), b.size(2), a.stride(0), b.stride(0), b.size(1),
-               (int)block_m, (int)top_k, mul_routed_weight ? 1 : 0, dtype_code(a, op),
+               sorted_token_ids.numel(), n, k, a.stride(0), expert_stride, n, (int)block_m,
+               (int)top_k, mul_routed_weight ? 1 : 0,
+               b_packed ? SARATHI_MOE_B_PACKED : SARATHI_MOE_B_ROW_MAJOR, dtype_code(a, op),
                scope.stream),
            op);
 }
@@ -351,5 +364,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("moe_align_block_size_filled", &moe_align_block_size_filled,
         "moe_align_block_size that also writes the padding value into unused slots");
   m.def("moe_grouped_gemm", &moe_grouped_gemm,
-        "C[slot] = A[slot / top_k] @ B[expert(slot)]^T over moe_align_block_size's layout");
+        "C[slot] = A[slot / top_k] @ B[expert(slot)]^T over moe_align_block_size's layout",
+        pybind11::arg("a"), pybind11::arg("b"), pybind11::arg("c"), pybind11::arg("topk_weights"),
+        pybind11::arg("sorted_token_ids"), pybind11::arg("expert_ids"),
+        pybind11::arg("num_tokens_post_padded"), pybind11::arg("num_valid_tokens"),
+        pybind11::arg("block_m"), pybind11::arg("top_k"), pybind11::arg("mul_routed_weight"),
+        pybind11::arg("b_packed") = false, pybind11::arg("n") = 0);
 }

@@ -3,7 +3,8 @@
 layers/fused_moe/fused_moe.py).  Same class / function names and call signatures, so model code written
 against the reference's layers runs unchanged; the bodies call this package's HIP ops."""
 from .activation import FastGELU, NewGELU, SiluAndMul, get_act_fn
-from .fused_moe import fused_experts, fused_moe, invoke_fused_moe_kernel
+from .fused_moe import (PackedExpertWeights, fused_experts, fused_moe, invoke_fused_moe_kernel,
+                        pack_expert_weights)
 from .moe_routing import fused_topk, moe_align_block_size
 from .norm import RMSNorm
 from .rotary import (DynamicNTKScalingRotaryEmbedding, LinearScalingRotaryEmbedding,
@@ -12,4 +13,5 @@ from .rotary import (DynamicNTKScalingRotaryEmbedding, LinearScalingRotaryEmbedd
 __all__ = ["RMSNorm", "SiluAndMul", "NewGELU", "FastGELU", "get_act_fn", "RotaryEmbedding",
            "LinearScalingRotaryEmbedding", "DynamicNTKScalingRotaryEmbedding",
            "YaRNScalingRotaryEmbedding", "get_rope", "fused_topk", "moe_align_block_size",
-           "invoke_fused_moe_kernel", "fused_experts", "fused_moe"]
+           "invoke_fused_moe_kernel", "fused_experts", "fused_moe", "pack_expert_weights",
+           "PackedExpertWeights"]

@@ -57,6 +57,14 @@ def test_grouped_gemm_matches_formulation(ops, dev, dtype, T, E, k, BM, N, K, mu
     ops.moe_ops.moe_grouped_gemm(A.to(dev), Bw.to(dev), got, w.to(dev), s.to(dev), e.to(dev),
                                  p.to(dev), T * k, BM, k, mul)
     _close(got, want, "grouped gemm")
+    # packed weight layout: same products, same accumulation order -> same bits
+    from sarathi_amd.layers import pack_expert_weights
+    packed = pack_expert_weights(Bw.to(dev))
+    assert packed.shape == (E, N, K)
+    got2 = torch.full((T, k, N), 7.0, dtype=dtype, device=dev)
+    ops.moe_ops.moe_grouped_gemm(A.to(dev), packed.data, got2, w.to(dev), s.to(dev), e.to(dev),
+                                 p.to(dev), T * k, BM, k, mul, True, N)
+    assert torch.equal(got2, got)
 
 
 def test_grouped_gemm_second_stage_addressing(ops, dev):
@@ -102,6 +110,10 @@ def test_fused_moe_forward(ops, dev, T, E, k, H, I, renorm):
     got = layers.fused_moe(x.to(dev), w1.to(dev), w2.to(dev), gating.to(dev), k, renorm)
     assert got.shape == (T, H) and got.dtype == torch.bfloat16
     _close(got, want, "fused_moe")
+    # packed expert weights give the same bits
+    p1, p2 = layers.pack_expert_weights(w1.to(dev)), layers.pack_expert_weights(w2.to(dev))
+    got_p = layers.fused_moe(x.to(dev), p1, p2, gating.to(dev), k, renorm)
+    assert torch.equal(got_p, got)
     # in place
     xd = x.to(dev)
     out = layers.fused_moe(xd, w1.to(dev), w2.to(dev), gating.to(dev), k, renorm, inplace=True)

@@ -494,3 +494,60 @@ def test_moe_align_id_dtypes(dtype):
     a = _align(c_oracle.moe_align_block_size, ids32, 100, 8)
     b = _align(c_oracle.moe_align_block_size, ids32.to(dtype), 100, 8)
     assert all(torch.equal(x, y) for x, y in zip(a, b))
+
+
+# ------------------------------------------------------- grouped expert GEMM
+
+def _routing(T, E, k, B, seed):
+    g = gen(seed)
+    gating = torch.randn((T, E), generator=g)
+    w, ids, _ = _topk(gating, k)
+    s, e, p = _align(c_oracle.moe_align_block_size, ids, E, B)
+    return gating, w, ids, s, e, p
+
+
+def test_grouped_gemm_formulation_brute_force():
+    """The tensor formulation of the reference's Triton kernel against a scalar float64 loop that
+    does not use the sorted layout at all: C[t, j] = w[t, j] * A[t] @ B[ids[t, j]]^T."""
+    T, E, k, B, N, K = 23, 4, 2, 8, 12, 16
+    _, w, ids, s, e, p = _routing(T, E, k, B, 60)
+    g = gen(61)
+    A = randn((T, K), g)
+    Bw = randn((E, N, K), g)
+    for mul in (False, True):
+        C = torch.full((T, k, N), 9.0, dtype=torch.bfloat16)
+        torch_formulations.moe_grouped_gemm(A, Bw, C, w, s, e, p, T * k, B, k, mul)
+        for t in range(T):
+            for j in range(k):
+                ref = A[t].double() @ Bw[int(ids[t, j])].double().t()
+                if mul:
+                    ref = ref * float(w[t, j])
+                assert torch.allclose(C[t, j].double(), ref, rtol=2 ** -7, atol=1e-6)
+    # every (token, j) row is written exactly once: no sentinel survives
+    assert not bool((C == 9.0).all(dim=-1).any())
+    # identity weights reproduce the token row exactly
+    eye = torch.stack([torch.eye(K)] * E).bfloat16()
+    C = torch.zeros((T, k, K), dtype=torch.bfloat16)
+    torch_formulations.moe_grouped_gemm(A, eye, C, w, s, e, p, T * k, B, k, False)
+    assert torch.equal(C, A.unsqueeze(1).expand(T, k, K))
+
+
+def test_fused_moe_formulation_against_float64_dense():
+    T, E, k, H, I = 40, 4, 2, 32, 48
+    g = gen(62)
+    x = randn((T, H), g)
+    w1 = randn((E, 2 * I, H), g, std=H ** -0.5)
+    w2 = randn((E, H, I), g, std=I ** -0.5)
+    gating = torch.randn((T, E), generator=g)
+    got = torch_formulations.fused_moe(x, w1, w2, gating, k, True)
+    p = torch.softmax(gating.double(), -1)
+    tw, ti = torch.topk(p, k, dim=-1)
+    tw = tw / tw.sum(-1, keepdim=True)
+    want = torch.zeros((T, H), dtype=torch.float64)
+    for t in range(T):
+        for j in range(k):
+            ex = int(ti[t, j])
+            gu = w1[ex].double() @ x[t].double()
+            h = torch.nn.functional.silu(gu[:I]) * gu[I:]
+            want[t] += tw[t, j] * (w2[ex].double() @ h)
+    assert torch.allclose(got.double(), want, rtol=3e-2, atol=3e-2 * want.abs().max().item())
