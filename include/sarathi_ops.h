@@ -173,7 +173,7 @@ int64_t sarathi_moe_align_workspace_bytes(int64_t numel, int num_experts);
  * [num_valid_tokens, N] with rows c_row_stride apart (num_valid_tokens =
  * tokens * topk; slots holding a larger id are padding and skipped).
  * block_m must be the block_size moe_align_block_size ran with and one of 32,
- * 64, 128; dtype bf16 or fp16; K a multiple of 64, N a multiple of 4.
+ * 64, 128, 256; dtype bf16 or fp16; K a multiple of 64, N a multiple of 4.
  *
  * b_layout: SARATHI_MOE_B_ROW_MAJOR is the reference's [E, N, K] tensor.
  * SARATHI_MOE_B_PACKED is the same weights re-tiled once, offline, into the

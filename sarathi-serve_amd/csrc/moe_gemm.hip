@@ -28,7 +28,7 @@
 //                coalesced load (~1.3-1.9x faster).  Weights are static, so
 //                packing them once at load time is free.
 //   tokens   shared by the four waves: gathered once per K-step into LDS
-//            (BM x 64 elements, 16-byte chunks XOR-swizzled by row so that the
+//            (BM x 64 elements, 16-byte chunks rotated by row so that the
 //            operand reads are bank-conflict free), double buffered, one
 //            barrier per K-step.
 // Workgroup ids are mapped so that the eight XCDs (id mod 8) each take their
@@ -56,6 +56,13 @@ template <int DT> SK_DEV f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
                                                   __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
+// Position (0..7) of 16-byte chunk c inside row r of the token tile in LDS.  Rows are 128 bytes,
+// i.e. exactly one pass over the 32 banks, so the bank group of an access is this position.
+// An operand read has lane (row r, half g) fetch chunk 2s + g; the rotation below makes the
+// positions distinct both over eight consecutive rows of one half and over four consecutive
+// rows of both halves, whichever way the hardware groups the lanes of a 128-bit read.
+SK_DEV int lds_slot(int r, int c) { return (c + 2 * (r & 3) + ((r >> 2) & 1)) & 7; }
+
 struct MoeGemmArgs {
   const void* a;            // [tokens, K]
   const void* b;            // [E, N, K]
@@ -74,13 +81,18 @@ struct MoeGemmArgs {
   int32_t m_blocks, n_blocks;
 };
 
-template <int DT, int BM, bool MUL_WEIGHT, bool PACKED>
-__global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmArgs g) {
-  constexpr int MT = BM / 32;          // token tiles per wave
+// BM slots per workgroup = WM wave rows x (BM / WM) slots; four wave columns of 64 output columns.
+// WM = 2 (BM = 256, eight waves) halves the number of times a weight tile is pulled out of L2,
+// which is what bounds this kernel once the loads are coalesced.
+template <int DT, int BM, int WM, bool MUL_WEIGHT, bool PACKED>
+__global__ __launch_bounds__(256 * WM) void moe_gemm_kernel(MoeGemmArgs g) {
+  constexpr int THREADS = 256 * WM;
+  constexpr int MT = BM / WM / 32;     // token tiles per wave
   constexpr int NT = kGemmWaveN / 32;  // weight tiles per wave
   constexpr int SUB = kGemmBK / 16;    // MFMA sub-steps per K-step
-  constexpr int A_LOADS = BM / 32;     // 16-byte chunks each thread gathers per K-step
-  __shared__ u32x4 tok_lds[2][BM * 8];  // [buffer][row * 8 + swizzled chunk]
+  constexpr int ROWS_PER_PASS = THREADS / 8;
+  constexpr int A_LOADS = BM / ROWS_PER_PASS;  // 16-byte chunks each thread gathers per K-step
+  __shared__ u32x4 tok_lds[2][BM * 8];  // [buffer][row * 8 + rotated chunk]
 
   // ---- which tile
   const unsigned id = blockIdx.x;
@@ -91,7 +103,9 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmArgs g) {
   if (pid_m * BM >= *g.num_tokens_post_padded) return;
   const int expert = g.expert_ids[pid_m];
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = (tid >> 6) & 3;          // wave column: output columns [64 wave, 64 wave + 64)
+  const int row0 = (tid >> 8) * (BM / WM);  // wave row: first slot of this wave inside the block
   const int l32 = lane & 31, grp = lane >> 5;
 
   // ---- weights: buffer resource over the expert's matrix; rows >= N read as zero
@@ -117,12 +131,12 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmArgs g) {
                   : buf_load16<kCached>(rb, w_off[nt] + (uint32_t)(k0 + s * 16) * 2u);
   };
 
-  // ---- tokens: each thread gathers chunk `tid & 7` of rows (tid >> 3) + 32 j
+  // ---- tokens: each thread gathers chunk `tid & 7` of rows (tid >> 3) + ROWS_PER_PASS j
   const int a_chunk = tid & 7;
   const char* a_ptr[A_LOADS];
 #pragma unroll
   for (int j = 0; j < A_LOADS; ++j) {
-    const int r = (tid >> 3) + 32 * j;
+    const int r = (tid >> 3) + ROWS_PER_PASS * j;
     const int slot_index = pid_m * BM + r;
     const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
     a_ptr[j] = sid < g.num_valid
@@ -138,8 +152,8 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmArgs g) {
   auto stage = [&](int buf, const u32x4 (&regs)[A_LOADS]) {
 #pragma unroll
     for (int j = 0; j < A_LOADS; ++j) {
-      const int r = (tid >> 3) + 32 * j;
-      tok_lds[buf][r * 8 + (a_chunk ^ (r & 7))] = regs[j];
+      const int r = (tid >> 3) + ROWS_PER_PASS * j;
+      tok_lds[buf][r * 8 + lds_slot(r, a_chunk)] = regs[j];
     }
   };
   f32x16 acc[NT][MT];
@@ -172,8 +186,8 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmArgs g) {
   auto read_tokens = [&](int buf, int s, u32x4 (&tokv)[MT]) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      const int r = mt * 32 + l32;
-      tokv[mt] = tok_lds[buf][r * 8 + ((2 * s + grp) ^ (r & 7))];
+      const int r = row0 + mt * 32 + l32;
+      tokv[mt] = tok_lds[buf][r * 8 + lds_slot(r, 2 * s + grp)];
     }
   };
   for (int step = 0; step < steps; ++step) {
@@ -206,7 +220,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmArgs g) {
   // ---- epilogue: lane holds, per accumulator quad, 4 consecutive columns of one token
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const int slot_index = pid_m * BM + mt * 32 + l32;
+    const int slot_index = pid_m * BM + row0 + mt * 32 + l32;
     const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
     if (sid >= g.num_valid) continue;
     float scale = 1.f;
@@ -236,12 +250,13 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmArgs g) {
 
 template <int DT, int BM>
 static int launch_moe_gemm(const MoeGemmArgs& g, bool mul_weight, bool packed, hipStream_t st) {
+  constexpr int WM = BM > 128 ? 2 : 1;
   const int64_t groups = (g.n_blocks + 7) / 8;
   const int64_t blocks = groups * g.m_blocks * 8;
   if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
-  const dim3 grid((unsigned)blocks), block(256);
+  const dim3 grid((unsigned)blocks), block(256 * WM);
 #define SK_LAUNCH(MW, PK) \
-  hipLaunchKernelGGL((moe_gemm_kernel<DT, BM, MW, PK>), grid, block, 0, st, g)
+  hipLaunchKernelGGL((moe_gemm_kernel<DT, BM, WM, MW, PK>), grid, block, 0, st, g)
   if (mul_weight) { if (packed) SK_LAUNCH(true, true); else SK_LAUNCH(true, false); }
   else { if (packed) SK_LAUNCH(false, true); else SK_LAUNCH(false, false); }
 #undef SK_LAUNCH
@@ -270,7 +285,8 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
     return SARATHI_ERR_INVALID_ARG;
   const bool packed = b_layout == SARATHI_MOE_B_PACKED;
   if (packed && b_expert_stride < (n + 31) / 32 * 32 * k) return SARATHI_ERR_INVALID_ARG;
-  if (block_m != 32 && block_m != 64 && block_m != 128) return SARATHI_ERR_UNSUPPORTED;
+  if (block_m != 32 && block_m != 64 && block_m != 128 && block_m != 256)
+    return SARATHI_ERR_UNSUPPORTED;
   if (dtype != kBF16 && dtype != kF16) return SARATHI_ERR_UNSUPPORTED;
   // 16-byte operand pieces and whole K-steps; one buffer resource per expert matrix
   if (k % kGemmBK != 0 || a_row_stride % 8 != 0 || b_expert_stride % 8 != 0 || n % 4 != 0 ||
@@ -300,7 +316,8 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
   switch (block_m) {                                                      \
     case 32: return launch_moe_gemm<DT, 32>(g, mw, packed, st);           \
     case 64: return launch_moe_gemm<DT, 64>(g, mw, packed, st);           \
-    default: return launch_moe_gemm<DT, 128>(g, mw, packed, st);          \
+    case 128: return launch_moe_gemm<DT, 128>(g, mw, packed, st);         \
+    default: return launch_moe_gemm<DT, 256>(g, mw, packed, st);          \
   }
   if (dtype == kBF16) { SK_GEMM(kBF16) } else { SK_GEMM(kF16) }
 #undef SK_GEMM

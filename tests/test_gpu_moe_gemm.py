@@ -43,6 +43,8 @@ def _close(got, want, what):
     (300, 8, 2, 64, 512, 256, True),
     (77, 4, 2, 32, 260, 128, True),      # N not a multiple of the 256-wide tile nor of 32
     (1000, 8, 2, 128, 768, 512, False),
+    (1500, 4, 2, 256, 512, 256, True),   # eight-wave tile
+    (40, 8, 2, 256, 300, 128, False),    # mostly padding
     (33, 16, 4, 32, 256, 64, True),      # some experts empty, single K step
     (5, 8, 1, 32, 1024, 192, False),
 ])
