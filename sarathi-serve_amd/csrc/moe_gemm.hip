@@ -71,6 +71,7 @@ struct MoeGemmArgs {
   const int32_t* sorted_token_ids;  // [em]
   const int32_t* expert_ids;        // [ceil(em / BM)]
   const int32_t* num_tokens_post_padded;
+  uint32_t a_bytes;         // extent of A in bytes (< 2 GiB)
   int64_t a_row_stride;     // elements
   int64_t b_expert_stride;  // elements
   int64_t c_row_stride;     // elements
@@ -131,23 +132,24 @@ __global__ __launch_bounds__(256 * WM) void moe_gemm_kernel(MoeGemmArgs g) {
                   : buf_load16<kCached>(rb, w_off[nt] + (uint32_t)(k0 + s * 16) * 2u);
   };
 
-  // ---- tokens: each thread gathers chunk `tid & 7` of rows (tid >> 3) + ROWS_PER_PASS j
+  // ---- tokens: each thread gathers chunk `tid & 7` of rows (tid >> 3) + ROWS_PER_PASS j.
+  // A is one buffer resource; padding slots get an offset beyond it, so their loads return
+  // zeros without a branch.
+  const rsrc_t ra = make_rsrc(g.a, g.a_bytes);
   const int a_chunk = tid & 7;
-  const char* a_ptr[A_LOADS];
+  uint32_t a_off[A_LOADS];
 #pragma unroll
   for (int j = 0; j < A_LOADS; ++j) {
     const int r = (tid >> 3) + ROWS_PER_PASS * j;
     const int slot_index = pid_m * BM + r;
     const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
-    a_ptr[j] = sid < g.num_valid
-                   ? reinterpret_cast<const char*>(g.a) + ((int64_t)(sid / g.top_k) * g.a_row_stride) * 2 + a_chunk * 16
-                   : nullptr;
+    a_off[j] = sid < g.num_valid
+                   ? (uint32_t)(sid / g.top_k) * (uint32_t)(g.a_row_stride * 2) + a_chunk * 16u
+                   : 0x80000000u;
   }
   auto gather = [&](int k0, u32x4 (&regs)[A_LOADS]) {
 #pragma unroll
-    for (int j = 0; j < A_LOADS; ++j)
-      regs[j] = a_ptr[j] ? *reinterpret_cast<const u32x4*>(a_ptr[j] + (int64_t)k0 * 2)
-                         : (u32x4){0, 0, 0, 0};
+    for (int j = 0; j < A_LOADS; ++j) regs[j] = buf_load16<kCached>(ra, a_off[j] + (uint32_t)k0 * 2u);
   };
   auto stage = [&](int buf, const u32x4 (&regs)[A_LOADS]) {
 #pragma unroll
@@ -294,6 +296,10 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
     return SARATHI_ERR_UNSUPPORTED;
   if ((n + 31) / 32 * 32 * k * 2 >= 0x80000000LL || num_valid_tokens > 0x7fffffffLL || sorted_len > 0x7fffffffLL)
     return SARATHI_ERR_UNSUPPORTED;
+  // A is addressed through one buffer resource with 32-bit offsets
+  const int64_t a_rows = (num_valid_tokens + top_k - 1) / top_k;
+  const int64_t a_extent = ((a_rows > 0 ? a_rows - 1 : 0) * a_row_stride + k) * 2;
+  if (a_extent >= 0x80000000LL) return SARATHI_ERR_UNSUPPORTED;
   if (sorted_len == 0 || num_valid_tokens == 0) return SARATHI_OK;
   MoeGemmArgs g;
   g.a = a; g.b = b; g.c = c;
@@ -301,6 +307,7 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
   g.sorted_token_ids = sorted_token_ids;
   g.expert_ids = expert_ids;
   g.num_tokens_post_padded = num_tokens_post_padded;
+  g.a_bytes = (uint32_t)a_extent;
   g.a_row_stride = a_row_stride;
   g.b_expert_stride = b_expert_stride;
   g.c_row_stride = c_row_stride;

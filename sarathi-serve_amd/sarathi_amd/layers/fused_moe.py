@@ -53,7 +53,7 @@ def get_default_config(M: int, E: int, N: int, K: int, topk: int,
     taller tile re-uses each weight fragment for more tokens).  BLOCK_SIZE_N / BLOCK_SIZE_K are
     fixed properties of the kernel and reported for information."""
     per_expert = M * topk / max(E, 1)
-    block_m = 256 if per_expert >= 768 else 128 if per_expert >= 384 else 64 if per_expert >= 96 else 32
+    block_m = 128 if per_expert >= 384 else 64 if per_expert >= 96 else 32   # 256 measured no faster
     return {"BLOCK_SIZE_M": block_m, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 64, "GROUP_SIZE_M": 1}
 
 
