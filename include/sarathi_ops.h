@@ -192,6 +192,61 @@ int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c, const float*
                              int top_k, int mul_routed_weight, int b_layout, int dtype,
                              void* stream);
 
+/*
+ * Paged KV cache (NHD page layout: entry e of page p holds [num_kv_heads, head_size] elements and
+ * starts page_stride*p + entry_stride*e elements after k_cache, resp. v_cache; the reference's
+ * cache tensor [num_pages, 2, page_size, num_kv_heads, head_size],
+ * sarathi/model_executor/attention/flashinfer_attention_wrapper.py:70-78, has k_cache = cache,
+ * v_cache = cache + page_size*num_kv_heads*head_size, page_stride = 2*page_size*num_kv_heads*
+ * head_size, entry_stride = num_kv_heads*head_size).
+ *
+ * The three calls below replace the flashinfer (flashinfer-python==0.4.1, requirements.txt:18)
+ * functions the reference's attention wrapper calls.
+ *
+ * sarathi_get_seq_lens replaces get_seq_lens (flashinfer_attention_wrapper.py:213-217):
+ *   seq_lens[i] = max(kv_indptr[i+1] - kv_indptr[i] - 1, 0) * page_size + kv_last_page_len[i].
+ * sarathi_get_batch_indices_positions replaces get_batch_indices_positions
+ * (flashinfer_attention_wrapper.py:220-226): for every request b and token i in
+ * [append_indptr[b], append_indptr[b+1]): batch_indices[i] = b and positions[i] =
+ * i + seq_lens[b] - append_indptr[b+1] (the request's last appended token is its last kv entry).
+ * Tokens outside [append_indptr[0], append_indptr[num_seqs]) are left untouched.
+ * sarathi_append_paged_kv_cache replaces append_paged_kv_cache(..., kv_layout="NHD")
+ * (flashinfer_attention_wrapper.py:262-273): token i's key and value rows are copied to entry
+ * positions[i] % page_size of page kv_indices[kv_indptr[batch_indices[i]] + positions[i] /
+ * page_size].  Indices are not range-checked.
+ */
+int sarathi_get_seq_lens(const int32_t* kv_indptr, const int32_t* kv_last_page_len,
+                         int32_t* seq_lens, int64_t num_seqs, int page_size, void* stream);
+int sarathi_get_batch_indices_positions(const int32_t* append_indptr, const int32_t* seq_lens,
+                                        int32_t* batch_indices, int32_t* positions,
+                                        int64_t num_seqs, int64_t nnz, void* stream);
+int sarathi_append_paged_kv_cache(const void* append_key, const void* append_value,
+                                  const int32_t* batch_indices, const int32_t* positions,
+                                  void* k_cache, void* v_cache, const int32_t* kv_indices,
+                                  const int32_t* kv_indptr, int64_t nnz, int num_kv_heads,
+                                  int head_size, int page_size, int64_t key_stride,
+                                  int64_t value_stride, int64_t page_stride, int64_t entry_stride,
+                                  int dtype, void* stream);
+
+/*
+ * New entry: sarathi_rotary_embedding followed by sarathi_append_paged_kv_cache in one launch,
+ * i.e. the reference's rotary call (sarathi/model_executor/models/llama.py:178) plus the cache
+ * append of the attention wrapper (flashinfer_attention_wrapper.py:262-273).  query is rotated in
+ * place for all num_tokens rows; the first num_append_tokens rows' rotated keys and their values
+ * are written to the cache (the reference appends key[:num_total_tokens]).  key itself is
+ * rotated in place only when write_key != 0 (attention reads keys from the cache, so the
+ * in-place result is normally dead) or for rows at or above num_append_tokens.  Results in
+ * query / key / cache are bit-identical to the two separate calls.
+ */
+int sarathi_rotary_embedding_append_paged_kv(
+    const int64_t* positions, void* query, void* key, const void* value, const void* cos_sin_cache,
+    const int32_t* batch_indices, const int32_t* append_positions, void* k_cache, void* v_cache,
+    const int32_t* kv_indices, const int32_t* kv_indptr, int64_t num_tokens,
+    int64_t num_append_tokens, int num_heads, int num_kv_heads, int head_size, int rot_dim,
+    int64_t query_stride, int64_t key_stride, int64_t value_stride, int page_size,
+    int64_t page_stride, int64_t entry_stride, int is_neox, int write_key, int dtype,
+    void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,42 @@
+// Where an appended token lands in a paged KV cache (NHD page layout).
+//
+// Follows the published algorithm of flashinfer's append_paged_kv_cache (the reference pins
+// flashinfer-python==0.4.1 in requirements.txt and calls it at
+// sarathi/model_executor/attention/flashinfer_attention_wrapper.py:262-273): token i belongs to
+// request b = batch_indices[i] and is the positions[i]-th entry of that request's key/value
+// sequence; the request's pages are kv_indices[kv_indptr[b] .. kv_indptr[b+1]), page_size entries
+// each, so the token goes to entry positions[i] % page_size of page
+// kv_indices[kv_indptr[b] + positions[i] / page_size].
+#pragma once
+
+#include <stdint.h>
+
+#include "vec16.h"
+
+namespace sarathi_hip {
+
+struct KvDest {
+  const int32_t* batch_indices;  // [nnz]
+  const int32_t* positions;      // [nnz] index of the token inside its request's kv sequence
+  const int32_t* kv_indices;     // page numbers, ragged over requests
+  const int32_t* kv_indptr;      // [requests + 1]
+  void* k_cache;                 // entry (page, e) of K starts at page*page_stride + e*entry_stride
+  void* v_cache;                 // same geometry for V
+  int64_t page_stride_bytes;
+  int64_t entry_stride_bytes;
+  int64_t nnz;                   // tokens to append (tokens at or above it are not appended)
+  int32_t page_size;
+};
+
+// Byte offset of token `tok`'s entry from k_cache / v_cache.  `tok` is uniform over the wave, so
+// the four dependent loads are scalar loads.
+SK_DEV int64_t kv_entry_offset(const KvDest& d, int64_t tok) {
+  const int32_t b = d.batch_indices[tok];
+  const uint32_t pos = (uint32_t)d.positions[tok];
+  const uint32_t pg = pos / (uint32_t)d.page_size;
+  const uint32_t entry = pos - pg * (uint32_t)d.page_size;
+  const int64_t page = d.kv_indices[(int64_t)d.kv_indptr[b] + pg];
+  return page * d.page_stride_bytes + (int64_t)entry * d.entry_stride_bytes;
+}
+
+}  // namespace sarathi_hip

@@ -71,7 +71,7 @@ struct MoeGemmArgs {
   const int32_t* sorted_token_ids;  // [em]
   const int32_t* expert_ids;        // [ceil(em / BM)]
   const int32_t* num_tokens_post_padded;
-  uint32_t a_bytes;         // extent of A in bytes (< 2 GiB)
+  uint32_t a_bytes;         // extent of A in bytes; a_bytes + 2*K stays below 4 GiB
   int64_t a_row_stride;     // elements
   int64_t b_expert_stride;  // elements
   int64_t c_row_stride;     // elements
@@ -133,8 +133,8 @@ __global__ __launch_bounds__(256 * WM) void moe_gemm_kernel(MoeGemmArgs g) {
   };
 
   // ---- tokens: each thread gathers chunk `tid & 7` of rows (tid >> 3) + ROWS_PER_PASS j.
-  // A is one buffer resource; padding slots get an offset beyond it, so their loads return
-  // zeros without a branch.
+  // A is one buffer resource; padding slots get an offset at its end (every K offset added
+  // later keeps them beyond it without wrapping), so their loads return zeros without a branch.
   const rsrc_t ra = make_rsrc(g.a, g.a_bytes);
   const int a_chunk = tid & 7;
   uint32_t a_off[A_LOADS];
@@ -145,7 +145,7 @@ __global__ __launch_bounds__(256 * WM) void moe_gemm_kernel(MoeGemmArgs g) {
     const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
     a_off[j] = sid < g.num_valid
                    ? (uint32_t)(sid / g.top_k) * (uint32_t)(g.a_row_stride * 2) + a_chunk * 16u
-                   : 0x80000000u;
+                   : g.a_bytes;
   }
   auto gather = [&](int k0, u32x4 (&regs)[A_LOADS]) {
 #pragma unroll
@@ -299,7 +299,7 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
   // A is addressed through one buffer resource with 32-bit offsets
   const int64_t a_rows = (num_valid_tokens + top_k - 1) / top_k;
   const int64_t a_extent = ((a_rows > 0 ? a_rows - 1 : 0) * a_row_stride + k) * 2;
-  if (a_extent >= 0x80000000LL) return SARATHI_ERR_UNSUPPORTED;
+  if (a_extent + 2 * k >= 0x100000000LL) return SARATHI_ERR_UNSUPPORTED;
   if (sorted_len == 0 || num_valid_tokens == 0) return SARATHI_OK;
   MoeGemmArgs g;
   g.a = a; g.b = b; g.c = c;

@@ -186,6 +186,174 @@ void rotary_embedding(torch::Tensor& positions, torch::Tensor& query, torch::Ten
            op);
 }
 
+// ---- kv_cache_ops --------------------------------------------------------------
+
+void check_i32(const torch::Tensor& t, const torch::Tensor& like, const char* op,
+               const char* name) {
+  check_gpu(t, like, op, name);
+  TORCH_CHECK(t.scalar_type() == at::ScalarType::Int && t.dim() == 1 && t.is_contiguous(), op,
+              ": ", name, " must be a contiguous int32 vector");
+}
+
+// k_cache / v_cache: [num_pages, page_size, num_kv_heads, head_size] views with the same strides
+struct PagedGeom {
+  int64_t page_size, heads, head_size, page_stride, entry_stride;
+};
+PagedGeom paged_geom(const torch::Tensor& k_cache, const torch::Tensor& v_cache, const char* op) {
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4, op,
+              ": k_cache and v_cache must be [num_pages, page_size, num_kv_heads, head_size]");
+  TORCH_CHECK(k_cache.sizes() == v_cache.sizes() && k_cache.strides() == v_cache.strides() &&
+                  k_cache.scalar_type() == v_cache.scalar_type(),
+              op, ": k_cache and v_cache must agree in shape, strides and dtype");
+  TORCH_CHECK(k_cache.stride(3) == 1 && k_cache.stride(2) == k_cache.size(3), op,
+              ": the [num_kv_heads, head_size] part of a cache entry must be contiguous");
+  return {k_cache.size(1), k_cache.size(2), k_cache.size(3), k_cache.stride(0), k_cache.stride(1)};
+}
+
+// rows of a [n, heads*head_size] or [n, heads, head_size] tensor: returns the row stride
+int64_t token_rows(const torch::Tensor& t, int64_t width, int64_t head_size, const char* op,
+                   const char* name) {
+  TORCH_CHECK(t.dim() == 2 || t.dim() == 3, op, ": ", name, " must be 2-D or 3-D");
+  if (t.dim() == 2) {
+    TORCH_CHECK(t.size(1) == width && t.stride(1) == 1, op, ": ", name, " rows must be ", width,
+                " contiguous elements");
+  } else {
+    TORCH_CHECK(t.size(1) * t.size(2) == width && t.size(2) == head_size && t.stride(2) == 1 &&
+                    t.stride(1) == head_size,
+                op, ": ", name, " must be [n, heads, ", head_size, "] with contiguous rows");
+  }
+  return t.stride(0);
+}
+
+void get_seq_lens(torch::Tensor& kv_indptr, torch::Tensor& kv_last_page_len,
+                  torch::Tensor& seq_lens, int64_t page_size) {
+  const char* op = "get_seq_lens";
+  check_i32(kv_indptr, kv_indptr, op, "kv_indptr");
+  check_i32(kv_last_page_len, kv_indptr, op, "kv_last_page_len");
+  check_i32(seq_lens, kv_indptr, op, "seq_lens");
+  const int64_t n = kv_last_page_len.numel();
+  TORCH_CHECK(kv_indptr.numel() == n + 1 && seq_lens.numel() == n && page_size > 0, op,
+              ": expected kv_indptr [n+1], kv_last_page_len [n], seq_lens [n]");
+  LaunchScope scope(kv_indptr);
+  raise_on(sarathi_get_seq_lens(kv_indptr.data_ptr<int32_t>(), kv_last_page_len.data_ptr<int32_t>(),
+                                seq_lens.data_ptr<int32_t>(), n, (int)page_size, scope.stream),
+           op);
+}
+
+void get_batch_indices_positions(torch::Tensor& append_indptr, torch::Tensor& seq_lens,
+                                 torch::Tensor& batch_indices, torch::Tensor& positions) {
+  const char* op = "get_batch_indices_positions";
+  check_i32(append_indptr, append_indptr, op, "append_indptr");
+  check_i32(seq_lens, append_indptr, op, "seq_lens");
+  check_i32(batch_indices, append_indptr, op, "batch_indices");
+  check_i32(positions, append_indptr, op, "positions");
+  const int64_t n = seq_lens.numel();
+  TORCH_CHECK(append_indptr.numel() == n + 1 && batch_indices.numel() == positions.numel(), op,
+              ": expected append_indptr [n+1], seq_lens [n], batch_indices and positions [nnz]");
+  LaunchScope scope(append_indptr);
+  raise_on(sarathi_get_batch_indices_positions(
+               append_indptr.data_ptr<int32_t>(), seq_lens.data_ptr<int32_t>(),
+               batch_indices.data_ptr<int32_t>(), positions.data_ptr<int32_t>(), n,
+               positions.numel(), scope.stream),
+           op);
+}
+
+void append_paged_kv_cache(torch::Tensor& append_key, torch::Tensor& append_value,
+                           torch::Tensor& batch_indices, torch::Tensor& positions,
+                           torch::Tensor& k_cache, torch::Tensor& v_cache,
+                           torch::Tensor& kv_indices, torch::Tensor& kv_indptr) {
+  const char* op = "append_paged_kv_cache";
+  check_gpu(append_key, append_key, op, "append_key");
+  check_gpu(append_value, append_key, op, "append_value");
+  check_gpu(k_cache, append_key, op, "k_cache");
+  check_gpu(v_cache, append_key, op, "v_cache");
+  check_i32(batch_indices, append_key, op, "batch_indices");
+  check_i32(positions, append_key, op, "positions");
+  check_i32(kv_indices, append_key, op, "kv_indices");
+  check_i32(kv_indptr, append_key, op, "kv_indptr");
+  const PagedGeom g = paged_geom(k_cache, v_cache, op);
+  TORCH_CHECK(append_key.scalar_type() == k_cache.scalar_type() &&
+                  append_value.scalar_type() == k_cache.scalar_type(),
+              op, ": keys, values and the cache must share a dtype");
+  const int64_t width = g.heads * g.head_size;
+  const int64_t ks = token_rows(append_key, width, g.head_size, op, "append_key");
+  const int64_t vs = token_rows(append_value, width, g.head_size, op, "append_value");
+  const int64_t nnz = append_key.size(0);
+  TORCH_CHECK(append_value.size(0) == nnz && batch_indices.numel() == nnz &&
+                  positions.numel() == nnz,
+              op, ": append_key, append_value, batch_indices and positions disagree on nnz");
+  LaunchScope scope(append_key);
+  raise_on(sarathi_append_paged_kv_cache(
+               append_key.data_ptr(), append_value.data_ptr(), batch_indices.data_ptr<int32_t>(),
+               positions.data_ptr<int32_t>(), k_cache.data_ptr(), v_cache.data_ptr(),
+               kv_indices.data_ptr<int32_t>(), kv_indptr.data_ptr<int32_t>(), nnz, (int)g.heads,
+               (int)g.head_size, (int)g.page_size, nnz > 1 ? ks : width, nnz > 1 ? vs : width,
+               g.page_stride, g.entry_stride, dtype_code(append_key, op), scope.stream),
+           op);
+}
+
+void rotary_embedding_append_paged_kv(torch::Tensor& positions, torch::Tensor& query,
+                                      torch::Tensor& key, torch::Tensor& value, int64_t head_size,
+                                      torch::Tensor& cos_sin_cache, bool is_neox,
+                                      torch::Tensor& batch_indices,
+                                      torch::Tensor& append_positions, torch::Tensor& k_cache,
+                                      torch::Tensor& v_cache, torch::Tensor& kv_indices,
+                                      torch::Tensor& kv_indptr, int64_t num_append_tokens,
+                                      bool write_key) {
+  const char* op = "rotary_embedding_append_paged_kv";
+  check_gpu(query, query, op, "query");
+  check_gpu(key, query, op, "key");
+  check_gpu(value, query, op, "value");
+  check_gpu(positions, query, op, "positions");
+  check_gpu(cos_sin_cache, query, op, "cos_sin_cache");
+  check_gpu(k_cache, query, op, "k_cache");
+  check_gpu(v_cache, query, op, "v_cache");
+  check_i32(batch_indices, query, op, "batch_indices");
+  check_i32(append_positions, query, op, "append_positions");
+  check_i32(kv_indices, query, op, "kv_indices");
+  check_i32(kv_indptr, query, op, "kv_indptr");
+  TORCH_CHECK(positions.scalar_type() == at::ScalarType::Long && positions.dim() == 1 &&
+                  positions.is_contiguous(),
+              op, ": positions must be a contiguous int64 [num_tokens] tensor");
+  TORCH_CHECK(query.dim() == 2 && key.dim() == 2 && value.dim() == 2, op,
+              ": query, key and value must be 2-D");
+  const int64_t T = positions.size(0);
+  TORCH_CHECK(query.size(0) == T && key.size(0) == T && value.size(0) == T, op,
+              ": query, key, value and positions disagree on num_tokens");
+  const PagedGeom g = paged_geom(k_cache, v_cache, op);
+  TORCH_CHECK(key.scalar_type() == query.scalar_type() &&
+                  value.scalar_type() == query.scalar_type() &&
+                  cos_sin_cache.scalar_type() == query.scalar_type() &&
+                  k_cache.scalar_type() == query.scalar_type(),
+              op, ": query, key, value, cos_sin_cache and the cache must share a dtype");
+  TORCH_CHECK(head_size == g.head_size && query.size(1) % head_size == 0 &&
+                  key.size(1) == g.heads * head_size && value.size(1) == key.size(1),
+              op, ": key / value rows must be num_kv_heads * head_size of the cache");
+  TORCH_CHECK(cos_sin_cache.dim() == 2 && cos_sin_cache.is_contiguous(), op,
+              ": cos_sin_cache must be a contiguous [max_position, rot_dim] tensor");
+  TORCH_CHECK(query.stride(1) == 1 && key.stride(1) == 1 && value.stride(1) == 1, op,
+              ": rows must be contiguous");
+  const int64_t rot_dim = cos_sin_cache.size(1);
+  TORCH_CHECK(rot_dim % 2 == 0 && rot_dim <= head_size, op,
+              ": rot_dim must be even and <= head_size");
+  TORCH_CHECK(num_append_tokens >= 0 && num_append_tokens <= T &&
+                  batch_indices.numel() >= num_append_tokens &&
+                  append_positions.numel() >= num_append_tokens,
+              op, ": num_append_tokens must be within num_tokens and the index vectors");
+  LaunchScope scope(query);
+  raise_on(sarathi_rotary_embedding_append_paged_kv(
+               positions.data_ptr<int64_t>(), query.data_ptr(), key.data_ptr(), value.data_ptr(),
+               cos_sin_cache.data_ptr(), batch_indices.data_ptr<int32_t>(),
+               append_positions.data_ptr<int32_t>(), k_cache.data_ptr(), v_cache.data_ptr(),
+               kv_indices.data_ptr<int32_t>(), kv_indptr.data_ptr<int32_t>(), T, num_append_tokens,
+               (int)(query.size(1) / head_size), (int)g.heads, (int)head_size, (int)rot_dim,
+               T > 1 ? query.stride(0) : query.size(1), T > 1 ? key.stride(0) : key.size(1),
+               T > 1 ? value.stride(0) : value.size(1), (int)g.page_size, g.page_stride,
+               g.entry_stride, is_neox ? 1 : 0, write_key ? 1 : 0, dtype_code(query, op),
+               scope.stream),
+           op);
+}
+
 // ---- moe_ops -----------------------------------------------------------------
 
 void topk_softmax_impl(torch::Tensor& topk_weights, torch::Tensor& topk_indices,
@@ -355,6 +523,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   // pos_encoding_ops
   m.def("rotary_embedding", &rotary_embedding,
         "in-place GPT-NeoX / GPT-J rotary embedding of query and key");
+  // kv_cache_ops
+  m.def("get_seq_lens", &get_seq_lens, "kv sequence lengths from the page table");
+  m.def("get_batch_indices_positions", &get_batch_indices_positions,
+        "request index and kv position of every appended token");
+  m.def("append_paged_kv_cache", &append_paged_kv_cache,
+        "copy key / value rows into their entries of a paged (NHD) KV cache");
+  m.def("rotary_embedding_append_paged_kv", &rotary_embedding_append_paged_kv,
+        "rotary_embedding fused with append_paged_kv_cache");
   // moe_ops
   m.def("topk_softmax", &topk_softmax, "softmax over experts + top-k (raw probabilities)");
   m.def("topk_softmax_renorm", &topk_softmax_renorm,

@@ -14,6 +14,10 @@ signatures (the reference builds them as four pybind11 modules, setup.py:95-136)
     moe_ops.moe_align_block_size(topk_ids, num_experts, block_size, sorted_token_ids,
                                  experts_ids, num_tokens_post_pad)
 
+``kv_cache_ops`` adds the paged KV-cache append that follows the rotary embedding on the
+reference's attention path (flashinfer's get_seq_lens / get_batch_indices_positions /
+append_paged_kv_cache signatures) and its fusion with rotary_embedding.
+
 All ops return None, write through out-parameters or in place, and launch
 asynchronously on torch's current stream.  There is no CPU or PyTorch fallback:
 importing this package raises ImportError when the compiled HIP extension is
@@ -21,6 +25,6 @@ missing.  ``sarathi_amd.layers`` holds counterparts of the reference's Python
 layer classes that call these ops.
 """
 from . import _ext  # noqa: F401  (raises ImportError if the HIP extension is not built)
-from . import activation_ops, layernorm_ops, moe_ops, pos_encoding_ops  # noqa: F401
+from . import activation_ops, kv_cache_ops, layernorm_ops, moe_ops, pos_encoding_ops  # noqa: F401
 
-__all__ = ["layernorm_ops", "activation_ops", "pos_encoding_ops", "moe_ops"]
+__all__ = ["layernorm_ops", "activation_ops", "pos_encoding_ops", "moe_ops", "kv_cache_ops"]

@@ -5,6 +5,7 @@ against the reference's layers runs unchanged; the bodies call this package's HI
 from .activation import FastGELU, NewGELU, SiluAndMul, get_act_fn
 from .fused_moe import (PackedExpertWeights, fused_experts, fused_moe, invoke_fused_moe_kernel,
                         pack_expert_weights)
+from .kv_append import AppendMetadata, SequenceSlice, build_append_metadata
 from .moe_routing import fused_topk, moe_align_block_size
 from .norm import RMSNorm
 from .rotary import (DynamicNTKScalingRotaryEmbedding, LinearScalingRotaryEmbedding,
@@ -14,4 +15,4 @@ __all__ = ["RMSNorm", "SiluAndMul", "NewGELU", "FastGELU", "get_act_fn", "Rotary
            "LinearScalingRotaryEmbedding", "DynamicNTKScalingRotaryEmbedding",
            "YaRNScalingRotaryEmbedding", "get_rope", "fused_topk", "moe_align_block_size",
            "invoke_fused_moe_kernel", "fused_experts", "fused_moe", "pack_expert_weights",
-           "PackedExpertWeights"]
+           "PackedExpertWeights", "SequenceSlice", "AppendMetadata", "build_append_metadata"]

@@ -44,7 +44,9 @@ def pack_expert_weights(w: torch.Tensor) -> PackedExpertWeights:
         w = torch.cat((w, w.new_zeros((E, n_pad - N, K))), dim=1)
     tiles = w.reshape(E, n_pad // 32, 32, K // 16, 2, 8).permute(0, 1, 3, 4, 2, 5).contiguous()
     return PackedExpertWeights(tiles, (E, N, K))
-CHUNK_SIZE = 64 * 1024     # tokens per pass, as in the reference (fused_moe.py:459)
+
+
+CHUNK_SIZE = 64 * 1024     # tokens per pass, as in the reference (fused_moe.py:437)
 
 
 def get_default_config(M: int, E: int, N: int, K: int, topk: int,
@@ -93,14 +95,19 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
     E, N, _ = w1.shape
     topk = topk_ids.shape[1]
     dev, dt = hidden_states.device, hidden_states.dtype
-    M = min(num_tokens, CHUNK_SIZE)
+    # the GEMM addresses its activations with 32-bit byte offsets: keep both inputs below 4 GiB
+    chunk = CHUNK_SIZE
+    eb = hidden_states.element_size()
+    while chunk > 1 and max(chunk * K, chunk * topk * (N // 2)) * eb + 4 * max(K, N) >= 1 << 32:
+        chunk //= 2
+    M = min(num_tokens, chunk)
     cache1 = torch.empty((M, topk, N), device=dev, dtype=dt)
     cache2 = torch.empty((M * topk, N // 2), device=dev, dtype=dt)
     cache3 = torch.empty((M, topk, w2.shape[1]), device=dev, dtype=dt)
     out = hidden_states if inplace else torch.empty_like(hidden_states)
     topk_weights = topk_weights.contiguous()
-    for begin in range(0, num_tokens, CHUNK_SIZE):
-        end = min(begin + CHUNK_SIZE, num_tokens)
+    for begin in range(0, num_tokens, chunk):
+        end = min(begin + chunk, num_tokens)
         n = end - begin
         cur_hidden = hidden_states[begin:end]
         cur_ids, cur_w = topk_ids[begin:end], topk_weights[begin:end]

@@ -135,3 +135,60 @@ def test_op_namespaces_match_the_reference_module_surface(ops):
     assert {"silu_and_mul", "gelu_new", "gelu_fast"} <= set(dir(ops.activation_ops))
     assert {"rotary_embedding"} <= set(dir(ops.pos_encoding_ops))
     assert {"topk_softmax", "moe_align_block_size"} <= set(dir(ops.moe_ops))
+
+
+def test_kv_cache_and_gemm_argument_validation_without_gpu(lib):
+    i64, ci, vp = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p
+    buf = ctypes.create_string_buffer(256)
+    p = ctypes.cast(buf, vp)
+    null = vp(None)
+    INVALID, UNSUPPORTED, OK = -1, -2, 0
+
+    def append(**kw):
+        return lib.sarathi_append_paged_kv_cache(
+            kw.get("key", p), p, p, p, p, kw.get("vc", p), p, p, i64(kw.get("nnz", 1)), ci(2),
+            ci(8), ci(kw.get("page", 4)), i64(kw.get("ks", 16)), i64(16),
+            i64(kw.get("ps", 64)), i64(kw.get("es", 16)), ci(kw.get("dt", 2)), null)
+    assert append(key=null) == INVALID
+    assert append(vc=null) == INVALID
+    assert append(ks=8) == INVALID        # key rows narrower than heads * head_size
+    assert append(es=8) == INVALID        # cache entries narrower than a row
+    assert append(ps=32) == INVALID       # page stride < page_size * entry stride
+    assert append(page=0) == INVALID
+    assert append(dt=6) == UNSUPPORTED
+    assert append(nnz=0) == OK
+
+    assert lib.sarathi_get_seq_lens(null, p, p, i64(1), ci(4), null) == INVALID
+    assert lib.sarathi_get_seq_lens(p, p, p, i64(1), ci(0), null) == INVALID
+    assert lib.sarathi_get_seq_lens(p, p, p, i64(0), ci(4), null) == OK
+    assert lib.sarathi_get_batch_indices_positions(p, p, null, p, i64(1), i64(1), null) == INVALID
+    assert lib.sarathi_get_batch_indices_positions(p, p, p, p, i64(0), i64(0), null) == OK
+
+    def fused(**kw):
+        return lib.sarathi_rotary_embedding_append_paged_kv(
+            kw.get("pos", p), p, p, kw.get("value", p), p, p, p, p, p, p, p, i64(kw.get("T", 1)),
+            i64(kw.get("n", 1)), ci(2), ci(1), ci(16), ci(kw.get("rot", 16)), i64(32),
+            i64(kw.get("ks", 16)), i64(16), ci(4), i64(64), i64(16), ci(1), ci(0),
+            ci(kw.get("dt", 2)), null)
+    assert fused(pos=null) == INVALID
+    assert fused(value=null) == INVALID
+    assert fused(n=2) == INVALID          # more appended tokens than tokens
+    assert fused(rot=18) == INVALID       # rot_dim > head_size
+    assert fused(ks=8) == INVALID
+    assert fused(dt=9) == UNSUPPORTED
+    assert fused(T=0, n=0) == OK
+
+    def gemm(**kw):
+        return lib.sarathi_moe_grouped_gemm(
+            kw.get("a", p), p, p, kw.get("w", p), p, p, p, i64(kw.get("valid", 4)), i64(64),
+            i64(kw.get("n", 64)), i64(kw.get("k", 64)), i64(kw.get("astride", 64)),
+            i64(64 * 128), i64(64), ci(kw.get("bm", 64)), ci(2), ci(kw.get("mul", 0)),
+            ci(kw.get("layout", 0)), ci(kw.get("dt", 2)), null)
+    assert gemm(a=null) == INVALID
+    assert gemm(w=null, mul=1) == INVALID           # routing weights required when multiplying
+    assert gemm(astride=32) == INVALID              # rows of A narrower than K
+    assert gemm(layout=5) == INVALID
+    assert gemm(bm=48) == UNSUPPORTED
+    assert gemm(dt=0) == UNSUPPORTED                # fp32 has no matrix-core path here
+    assert gemm(k=72, astride=72) == UNSUPPORTED    # K must be whole 64-wide steps
+    assert gemm(valid=0) == OK

@@ -173,7 +173,7 @@ def test_moe_align_skewed_and_empty(ops, dev):
 
 
 def test_moe_align_invariants_large(ops, dev):
-    """64K tokens x top-2 (the largest chunk the reference's caller passes, fused_moe.py:459):
+    """64K tokens x top-2 (the largest chunk the reference's caller passes, fused_moe.py:437):
     non-padding entries are a permutation of 0..numel-1, each block holds one expert's tokens in
     ascending order, post_pad = sum ceil(cnt/B)*B."""
     g = gen(12)

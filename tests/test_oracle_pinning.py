@@ -551,3 +551,88 @@ def test_fused_moe_formulation_against_float64_dense():
             h = torch.nn.functional.silu(gu[:I]) * gu[I:]
             want[t] += tw[t, j] * (w2[ex].double() @ h)
     assert torch.allclose(got.double(), want, rtol=3e-2, atol=3e-2 * want.abs().max().item())
+
+
+# ---- paged KV-cache append (oracle/paged_kv.py) ------------------------------------------------
+
+def _paged_case(seed, page_size, lens_before, new_tokens, heads=2, head_size=4, spare_pages=3):
+    """Random page tables for requests that already hold lens_before[i] tokens and get
+    new_tokens[i] more."""
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    totals = [a + b for a, b in zip(lens_before, new_tokens)]
+    need = [(t + page_size - 1) // page_size for t in totals]
+    num_pages = sum(need) + spare_pages
+    perm = rng.permutation(num_pages)
+    kv_indptr = np.concatenate([[0], np.cumsum(need)]).astype(np.int32)
+    kv_indices = perm[:sum(need)].astype(np.int32)
+    last = np.array([(t % page_size) or page_size if t > 0 else 0 for t in totals], dtype=np.int32)
+    append_indptr = np.concatenate([[0], np.cumsum(new_tokens)]).astype(np.int32)
+    nnz = int(append_indptr[-1])
+    k = rng.standard_normal((nnz, heads, head_size)).astype(np.float32)
+    v = rng.standard_normal((nnz, heads, head_size)).astype(np.float32)
+    cache = rng.standard_normal((num_pages, 2, page_size, heads, head_size)).astype(np.float32)
+    return dict(kv_indptr=kv_indptr, kv_indices=kv_indices, last=last, append_indptr=append_indptr,
+                nnz=nnz, k=k, v=v, cache=cache, totals=totals, page_size=page_size)
+
+
+def test_paged_kv_hand_worked_example():
+    """Two requests, page size 4.  Request 0 holds 5 tokens after getting 3 new ones (pages 7, 2);
+    request 1 is a decode step reaching 9 tokens (pages 0, 5, 3)."""
+    import numpy as np
+    from oracle import paged_kv
+    kv_indptr, kv_indices = [0, 2, 5], [7, 2, 0, 5, 3]
+    last = [1, 1]
+    seq_lens = paged_kv.get_seq_lens(kv_indptr, last, 4)
+    assert seq_lens.tolist() == [5, 9]
+    b, pos = paged_kv.get_batch_indices_positions([0, 3, 4], seq_lens, 4)
+    assert b.tolist() == [0, 0, 0, 1] and pos.tolist() == [2, 3, 4, 8]
+    cache = np.zeros((8, 2, 4, 1, 1), dtype=np.float32)
+    k = np.arange(1, 5, dtype=np.float32).reshape(4, 1, 1)
+    paged_kv.append_paged_kv_cache(k, -k, b, pos, cache[:, 0], cache[:, 1], kv_indices, kv_indptr)
+    want = {(7, 2): 1.0, (7, 3): 2.0, (2, 0): 3.0, (3, 0): 4.0}   # (page, entry) -> key value
+    for page in range(8):
+        for e in range(4):
+            assert cache[page, 0, e, 0, 0] == want.get((page, e), 0.0)
+            assert cache[page, 1, e, 0, 0] == -want.get((page, e), 0.0)
+
+
+@pytest.mark.parametrize("page_size,before,new", [
+    (4, [0, 0, 0], [1, 7, 8]),                # fresh prompts, lengths around page multiples
+    (16, [30, 16, 0, 5], [3, 1, 40, 1]),      # chunked prefill continuation + decodes
+    (1, [2, 0], [3, 2]),                      # page size 1
+    (8, [7, 8, 9], [1, 1, 1]),                # decode steps straddling a page boundary
+    (8, [3, 0, 11], [0, 5, 0]),               # requests with nothing to append
+])
+def test_paged_kv_round_trip_and_untouched_entries(page_size, before, new):
+    """Appending the new tokens after the old ones and gathering each request through its page
+    table returns old || new in order; every entry nobody wrote keeps its bytes."""
+    import numpy as np
+    from oracle import paged_kv
+    c = _paged_case(page_size + len(new), page_size, before, new)
+    seq_lens = paged_kv.get_seq_lens(c["kv_indptr"], c["last"], page_size)
+    assert seq_lens.tolist() == c["totals"]
+    b, pos = paged_kv.get_batch_indices_positions(c["append_indptr"], seq_lens, c["nnz"])
+    assert (b >= 0).all()
+    for r in range(len(new)):
+        lo, hi = c["append_indptr"][r], c["append_indptr"][r + 1]
+        assert (b[lo:hi] == r).all()
+        assert pos[lo:hi].tolist() == list(range(before[r], before[r] + new[r]))
+    cache = c["cache"].copy()
+    paged_kv.append_paged_kv_cache(c["k"], c["v"], b, pos, cache[:, 0], cache[:, 1],
+                                   c["kv_indices"], c["kv_indptr"])
+    written = np.zeros(cache.shape[:3], dtype=bool)
+    for r in range(len(new)):
+        lo, hi = c["append_indptr"][r], c["append_indptr"][r + 1]
+        for plane, src in ((0, c["k"]), (1, c["v"])):
+            got = paged_kv.gather_sequence(cache[:, plane], c["kv_indices"], c["kv_indptr"],
+                                           seq_lens, r)
+            old = paged_kv.gather_sequence(c["cache"][:, plane], c["kv_indices"], c["kv_indptr"],
+                                           seq_lens, r)
+            assert np.array_equal(got[before[r]:], src[lo:hi])
+            assert np.array_equal(got[:before[r]], old[:before[r]])
+        pages = c["kv_indices"][c["kv_indptr"][r]:c["kv_indptr"][r + 1]]
+        for j in range(before[r], before[r] + new[r]):
+            written[pages[j // page_size], :, j % page_size] = True
+    assert np.array_equal(cache[~written], c["cache"][~written])
+    assert not np.array_equal(cache[written], c["cache"][written]) or not written.any()
