@@ -50,6 +50,16 @@ BYTES = {
     "rotary_embedding": 2 * (T * NQ * D + T * NKV * D) * BF16 + T * 8 + T * D * BF16,
     "silu_and_mul": (2 * T * DFF + T * DFF) * BF16,
 }
+# the step after rotary_embedding on the reference path: k and v rows go to their paged-cache
+# entries (read once, written once; 16 index bytes per token) ...
+PAGE = 16
+BYTES["append_paged_kv_cache"] = 4 * T * NKV * D * BF16 + T * 16
+# ... and the fusion of the two: q read + written, k and v read once, cache entries written once
+BYTES["rotary_embedding_append_paged_kv"] = (2 * T * NQ * D + 4 * T * NKV * D) * BF16 + T * 24 + \
+    T * D * BF16
+BYTES["append_paged_kv_cache (slot mapping)"] = 4 * T * NKV * D * BF16 + T * 4
+BYTES["rotary_embedding_append_paged_kv (slot mapping)"] = \
+    BYTES["rotary_embedding_append_paged_kv"] - T * 12
 MOE_T, MOE_E, MOE_K, MOE_B = 4096, 8, 2, 64
 BYTES["topk_softmax"] = MOE_T * MOE_E * 4 + 3 * MOE_T * MOE_K * 4
 _moe_sorted = MOE_T * MOE_K + MOE_E * (MOE_B - 1)
@@ -148,7 +158,7 @@ def main():
 
     def ring(name, make):
         n = max(4, int(COLD_FOOTPRINT // BYTES[name]) + 1)
-        return [make() for _ in range(n)]
+        return [make() for _ in range(n)]          # a set may hold more than the op touches
 
     w_dev = sets[0]["w1"]
     cache_dev = sets[0]["cache"]
@@ -170,6 +180,40 @@ def main():
     def mk_silu():
         return (dev_randn((T, 2 * DFF)), torch.empty((T, DFF), dtype=torch.bfloat16, device=dev))
 
+    # paged KV cache of the hybrid batch: one prompt chunk continuing a 4096-token request and
+    # 256 decode requests with contexts of 1..3000 tokens, pages handed out in random order
+    from sarathi_amd import kv_cache_ops as KV
+    from sarathi_amd import layers as LAYERS
+    import numpy as np
+    rng = np.random.default_rng(5)
+    lens = [(True, PREFILL, 4096 + PREFILL)] + [(False, 1, int(c))
+                                                for c in rng.integers(1, 3000, size=T - PREFILL)]
+    need = [(t + PAGE - 1) // PAGE for _, _, t in lens]
+    perm = rng.permutation(sum(need))
+    seqs, at = [], 0
+    for (is_p, new, tot), n_pages in zip(lens, need):
+        seqs.append(LAYERS.SequenceSlice(is_p, new, tot, perm[at:at + n_pages].tolist()))
+        at += n_pages
+    meta = LAYERS.build_append_metadata(seqs, PAGE, dev)
+    assert meta.num_total_tokens == T
+    # every ring set gets its own cache of just the pages that are written (plus the old ones'
+    # numbers: entries are addressed through the page table, so the tensor must span them all)
+    touched = torch.unique((meta.append_kv_page_indices[
+        (meta.append_kv_page_indptr[meta.append_batch_indices.long()]
+         + meta.append_positions // PAGE).long()]).long())
+    remap = torch.zeros(sum(need), dtype=torch.int32, device=dev)
+    remap[touched] = torch.arange(touched.numel(), dtype=torch.int32, device=dev)
+    kv_indices_dense = remap[meta.append_kv_page_indices.long()]   # untouched pages alias page 0
+
+    slots_dense = KV.get_kv_slot_mapping(meta.append_batch_indices, meta.append_positions,
+                                         kv_indices_dense, meta.append_kv_page_indptr, PAGE)
+
+    def mk_kv():
+        qkv = dev_randn((T, (NQ + 2 * NKV) * D))
+        q, k, v = qkv.split([NQ * D, NKV * D, NKV * D], dim=-1)
+        cache = torch.empty((touched.numel(), 2, PAGE, NKV, D), dtype=torch.bfloat16, device=dev)
+        return (qkv, q, k, v, (cache[:, 0], cache[:, 1]))   # K / V planes split once, not per call
+
     mg = gen(3)
     gating = torch.randn((MOE_T, MOE_E), generator=mg, dtype=torch.float32).to(dev)
     tw = torch.empty((MOE_T, MOE_K), dtype=torch.float32, device=dev)
@@ -187,6 +231,26 @@ def main():
         "rotary_embedding": (ring("rotary_embedding", mk_rope),
                              lambda a: ROPE.rotary_embedding(pos_dev, a[1], a[2], D, cache_dev, True)),
         "silu_and_mul": (ring("silu_and_mul", mk_silu), lambda a: ACT.silu_and_mul(a[1], a[0])),
+        "append_paged_kv_cache": (ring("append_paged_kv_cache", mk_kv),
+                                  lambda a: KV.append_paged_kv_cache(
+                                      a[2], a[3], meta.append_batch_indices, meta.append_positions,
+                                      a[4], kv_indices_dense, meta.append_kv_page_indptr)),
+        "rotary_embedding_append_paged_kv": (
+            ring("rotary_embedding_append_paged_kv", mk_kv),
+            lambda a: KV.rotary_embedding_append_paged_kv(
+                pos_dev, a[1], a[2], a[3], D, cache_dev, True, meta.append_batch_indices,
+                meta.append_positions, a[4], kv_indices_dense, meta.append_kv_page_indptr)),
+        "append_paged_kv_cache (slot mapping)": (
+            ring("append_paged_kv_cache", mk_kv),
+            lambda a: KV.append_paged_kv_cache(
+                a[2], a[3], meta.append_batch_indices, meta.append_positions, a[4],
+                kv_indices_dense, meta.append_kv_page_indptr, slot_mapping=slots_dense)),
+        "rotary_embedding_append_paged_kv (slot mapping)": (
+            ring("rotary_embedding_append_paged_kv", mk_kv),
+            lambda a: KV.rotary_embedding_append_paged_kv(
+                pos_dev, a[1], a[2], a[3], D, cache_dev, True, meta.append_batch_indices,
+                meta.append_positions, a[4], kv_indices_dense, meta.append_kv_page_indptr,
+                slot_mapping=slots_dense)),
         "topk_softmax": ([None], lambda a: MOE.topk_softmax(tw, ti, ts, gating)),
         "moe_align_block_size": ([None], lambda a: MOE.moe_align_block_size_filled(
             ti, MOE_E, MOE_B, sorted_ids, expert_ids, post_pad)),

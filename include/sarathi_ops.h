@@ -214,7 +214,16 @@ int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c, const float*
  * (flashinfer_attention_wrapper.py:262-273): token i's key and value rows are copied to entry
  * positions[i] % page_size of page kv_indices[kv_indptr[batch_indices[i]] + positions[i] /
  * page_size].  Indices are not range-checked.
+ *
+ * sarathi_get_kv_slot_mapping (new) resolves that lookup once per batch:
+ * slot_mapping[i] = page * page_size + entry.  The page table of a batch is the same for every
+ * layer, so the append entry points accept the vector in place of the four index arrays
+ * (slot_mapping != NULL: batch_indices, positions, kv_indices and kv_indptr are ignored and may be
+ * NULL) and then need one index load per token instead of three dependent ones.
  */
+int sarathi_get_kv_slot_mapping(const int32_t* batch_indices, const int32_t* positions,
+                                const int32_t* kv_indices, const int32_t* kv_indptr,
+                                int32_t* slot_mapping, int64_t nnz, int page_size, void* stream);
 int sarathi_get_seq_lens(const int32_t* kv_indptr, const int32_t* kv_last_page_len,
                          int32_t* seq_lens, int64_t num_seqs, int page_size, void* stream);
 int sarathi_get_batch_indices_positions(const int32_t* append_indptr, const int32_t* seq_lens,
@@ -223,7 +232,8 @@ int sarathi_get_batch_indices_positions(const int32_t* append_indptr, const int3
 int sarathi_append_paged_kv_cache(const void* append_key, const void* append_value,
                                   const int32_t* batch_indices, const int32_t* positions,
                                   void* k_cache, void* v_cache, const int32_t* kv_indices,
-                                  const int32_t* kv_indptr, int64_t nnz, int num_kv_heads,
+                                  const int32_t* kv_indptr, const int32_t* slot_mapping,
+                                  int64_t nnz, int num_kv_heads,
                                   int head_size, int page_size, int64_t key_stride,
                                   int64_t value_stride, int64_t page_stride, int64_t entry_stride,
                                   int dtype, void* stream);
@@ -241,9 +251,9 @@ int sarathi_append_paged_kv_cache(const void* append_key, const void* append_val
 int sarathi_rotary_embedding_append_paged_kv(
     const int64_t* positions, void* query, void* key, const void* value, const void* cos_sin_cache,
     const int32_t* batch_indices, const int32_t* append_positions, void* k_cache, void* v_cache,
-    const int32_t* kv_indices, const int32_t* kv_indptr, int64_t num_tokens,
-    int64_t num_append_tokens, int num_heads, int num_kv_heads, int head_size, int rot_dim,
-    int64_t query_stride, int64_t key_stride, int64_t value_stride, int page_size,
+    const int32_t* kv_indices, const int32_t* kv_indptr, const int32_t* slot_mapping,
+    int64_t num_tokens, int64_t num_append_tokens, int num_heads, int num_kv_heads, int head_size,
+    int rot_dim, int64_t query_stride, int64_t key_stride, int64_t value_stride, int page_size,
     int64_t page_stride, int64_t entry_stride, int is_neox, int write_key, int dtype,
     void* stream);
 

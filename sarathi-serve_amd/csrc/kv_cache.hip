@@ -75,6 +75,19 @@ __global__ __launch_bounds__(256) void kv_batch_positions_kernel(
   positions[i] = (int32_t)(i + seq_lens[lo] - append_indptr[lo + 1]);
 }
 
+// slot_mapping[i] = page * page_size + entry of appended token i
+__global__ __launch_bounds__(256) void kv_slot_mapping_kernel(
+    const int32_t* __restrict__ batch_indices, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ kv_indices, const int32_t* __restrict__ kv_indptr,
+    int32_t* __restrict__ slot_mapping, int64_t nnz, int32_t page_size) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nnz) return;
+  const uint32_t pos = (uint32_t)positions[i];
+  const uint32_t pg = pos / (uint32_t)page_size;
+  const int32_t page = kv_indices[(int64_t)kv_indptr[batch_indices[i]] + pg];
+  slot_mapping[i] = page * page_size + (int32_t)(pos - pg * (uint32_t)page_size);
+}
+
 }  // namespace sarathi_hip
 
 using namespace sarathi_hip;
@@ -86,11 +99,11 @@ static int elem_bytes_of(int dtype) {
 extern "C" int sarathi_append_paged_kv_cache(
     const void* append_key, const void* append_value, const int32_t* batch_indices,
     const int32_t* positions, void* k_cache, void* v_cache, const int32_t* kv_indices,
-    const int32_t* kv_indptr, int64_t nnz, int num_kv_heads, int head_size, int page_size,
-    int64_t key_stride, int64_t value_stride, int64_t page_stride, int64_t entry_stride, int dtype,
-    void* stream) {
-  if (!append_key || !append_value || !batch_indices || !positions || !k_cache || !v_cache ||
-      !kv_indices || !kv_indptr)
+    const int32_t* kv_indptr, const int32_t* slot_mapping, int64_t nnz, int num_kv_heads,
+    int head_size, int page_size, int64_t key_stride, int64_t value_stride, int64_t page_stride,
+    int64_t entry_stride, int dtype, void* stream) {
+  if (!append_key || !append_value || !k_cache || !v_cache) return SARATHI_ERR_INVALID_ARG;
+  if (!slot_mapping && (!batch_indices || !positions || !kv_indices || !kv_indptr))
     return SARATHI_ERR_INVALID_ARG;
   const int64_t row = (int64_t)num_kv_heads * head_size;
   if (nnz < 0 || num_kv_heads <= 0 || head_size <= 0 || page_size <= 0 || key_stride < row ||
@@ -100,8 +113,9 @@ extern "C" int sarathi_append_paged_kv_cache(
   if (eb == 0 || row * eb >= 0x80000000LL || nnz > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
   if (nnz == 0) return SARATHI_OK;
   hipStream_t st = (hipStream_t)stream;
-  KvDest d{batch_indices, positions,          kv_indices, kv_indptr,     k_cache, v_cache,
-           page_stride * eb, entry_stride * eb, nnz,        (int32_t)page_size};
+  KvDest d{batch_indices, positions, kv_indices,       kv_indptr,         slot_mapping,
+           k_cache,       v_cache,   page_stride * eb, entry_stride * eb, nnz,
+           (int32_t)page_size};
   const uint32_t row_bytes = (uint32_t)(row * eb);
   const int64_t ksb = key_stride * eb, vsb = value_stride * eb;
   const bool vec_ok = row_bytes % 16 == 0 && ksb % 16 == 0 && vsb % 16 == 0 &&
@@ -121,8 +135,12 @@ extern "C" int sarathi_append_paged_kv_cache(
   if (rem > 0) {
     const int64_t t0 = full_z * kMaxGridY;
     KvDest dr = d;
-    dr.batch_indices += t0;
-    dr.positions += t0;
+    if (dr.slot_mapping) {
+      dr.slot_mapping += t0;
+    } else {
+      dr.batch_indices += t0;
+      dr.positions += t0;
+    }
     hipLaunchKernelGGL(kv_append_seg_kernel, dim3(2 * bpr, (unsigned)rem, 1), dim3(64), 0, st,
                        reinterpret_cast<const char*>(append_key) + t0 * ksb,
                        reinterpret_cast<const char*>(append_value) + t0 * vsb, ksb, vsb, row_bytes,
@@ -155,5 +173,20 @@ extern "C" int sarathi_get_batch_indices_positions(const int32_t* append_indptr,
   hipLaunchKernelGGL(kv_batch_positions_kernel, dim3((unsigned)((nnz + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, append_indptr, seq_lens, batch_indices, positions,
                      num_seqs, nnz);
+  return launch_status();
+}
+
+extern "C" int sarathi_get_kv_slot_mapping(const int32_t* batch_indices, const int32_t* positions,
+                                           const int32_t* kv_indices, const int32_t* kv_indptr,
+                                           int32_t* slot_mapping, int64_t nnz, int page_size,
+                                           void* stream) {
+  if (!batch_indices || !positions || !kv_indices || !kv_indptr || !slot_mapping || nnz < 0 ||
+      page_size <= 0)
+    return SARATHI_ERR_INVALID_ARG;
+  if (nnz == 0) return SARATHI_OK;
+  if (nnz > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(kv_slot_mapping_kernel, dim3((unsigned)((nnz + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, batch_indices, positions, kv_indices, kv_indptr,
+                     slot_mapping, nnz, (int32_t)page_size);
   return launch_status();
 }

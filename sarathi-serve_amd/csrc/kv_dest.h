@@ -20,6 +20,8 @@ struct KvDest {
   const int32_t* positions;      // [nnz] index of the token inside its request's kv sequence
   const int32_t* kv_indices;     // page numbers, ragged over requests
   const int32_t* kv_indptr;      // [requests + 1]
+  const int32_t* slot_mapping;   // optional [nnz]: page * page_size + entry, precomputed once per
+                                 // batch; replaces the three dependent lookups above
   void* k_cache;                 // entry (page, e) of K starts at page*page_stride + e*entry_stride
   void* v_cache;                 // same geometry for V
   int64_t page_stride_bytes;
@@ -31,6 +33,12 @@ struct KvDest {
 // Byte offset of token `tok`'s entry from k_cache / v_cache.  `tok` is uniform over the wave, so
 // the four dependent loads are scalar loads.
 SK_DEV int64_t kv_entry_offset(const KvDest& d, int64_t tok) {
+  if (d.slot_mapping != nullptr) {
+    const uint32_t slot = (uint32_t)d.slot_mapping[tok];
+    const uint32_t page = slot / (uint32_t)d.page_size;
+    const uint32_t entry = slot - page * (uint32_t)d.page_size;
+    return (int64_t)page * d.page_stride_bytes + (int64_t)entry * d.entry_stride_bytes;
+  }
   const int32_t b = d.batch_indices[tok];
   const uint32_t pos = (uint32_t)d.positions[tok];
   const uint32_t pg = pos / (uint32_t)d.page_size;

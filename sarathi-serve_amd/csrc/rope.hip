@@ -392,8 +392,12 @@ static int launch_rope_append(const RopeArgs& a, const void* value, int64_t v_st
   if (rem > 0) {
     const int64_t t0 = full_z * kMaxGridY;
     KvDest dr = d;
-    dr.batch_indices += t0;
-    dr.positions += t0;
+    if (dr.slot_mapping) {
+      dr.slot_mapping += t0;
+    } else {
+      dr.batch_indices += t0;
+      dr.positions += t0;
+    }
     dr.nnz = d.nnz > t0 ? d.nnz - t0 : 0;
     hipLaunchKernelGGL((rope_append_seg_kernel<DT, NEOX>), dim3(gx, (unsigned)rem, 1), dim3(64), 0,
                        st, reinterpret_cast<char*>(a.query) + t0 * qsb,
@@ -437,14 +441,15 @@ extern "C" int sarathi_rotary_embedding(const int64_t* positions, void* query, v
 extern "C" int sarathi_rotary_embedding_append_paged_kv(
     const int64_t* positions, void* query, void* key, const void* value, const void* cos_sin_cache,
     const int32_t* batch_indices, const int32_t* append_positions, void* k_cache, void* v_cache,
-    const int32_t* kv_indices, const int32_t* kv_indptr, int64_t num_tokens,
-    int64_t num_append_tokens, int num_heads, int num_kv_heads, int head_size, int rot_dim,
-    int64_t query_stride, int64_t key_stride, int64_t value_stride, int page_size,
+    const int32_t* kv_indices, const int32_t* kv_indptr, const int32_t* slot_mapping,
+    int64_t num_tokens, int64_t num_append_tokens, int num_heads, int num_kv_heads, int head_size,
+    int rot_dim, int64_t query_stride, int64_t key_stride, int64_t value_stride, int page_size,
     int64_t page_stride, int64_t entry_stride, int is_neox, int write_key, int dtype,
     void* stream) {
   using namespace sarathi_hip;
-  if (!positions || !query || !key || !value || !cos_sin_cache || !batch_indices ||
-      !append_positions || !k_cache || !v_cache || !kv_indices || !kv_indptr)
+  if (!positions || !query || !key || !value || !cos_sin_cache || !k_cache || !v_cache)
+    return SARATHI_ERR_INVALID_ARG;
+  if (!slot_mapping && (!batch_indices || !append_positions || !kv_indices || !kv_indptr))
     return SARATHI_ERR_INVALID_ARG;
   if (num_tokens < 0 || num_append_tokens < 0 || num_append_tokens > num_tokens ||
       num_heads <= 0 || num_kv_heads <= 0 || head_size <= 0 || rot_dim <= 0 || (rot_dim & 1) ||
@@ -459,8 +464,9 @@ extern "C" int sarathi_rotary_embedding_append_paged_kv(
   const int eb = dtype == kF32 ? 4 : 2;
   RopeArgs a{positions, query,     key,          cos_sin_cache, num_tokens, query_stride,
              key_stride, num_heads, num_kv_heads, head_size,     rot_dim};
-  KvDest d{batch_indices, append_positions,   kv_indices,        kv_indptr,        k_cache, v_cache,
-           page_stride * eb, entry_stride * eb, num_append_tokens, (int32_t)page_size};
+  KvDest d{batch_indices, append_positions, kv_indices,       kv_indptr,         slot_mapping,
+           k_cache,       v_cache,          page_stride * eb, entry_stride * eb, num_append_tokens,
+           (int32_t)page_size};
   hipStream_t st = (hipStream_t)stream;
 #define SK_ROPE_APPEND(DT)                                                              \
   (is_neox ? launch_rope_append<DT, true>(a, value, value_stride, write_key, d, st)     \

@@ -258,10 +258,33 @@ void get_batch_indices_positions(torch::Tensor& append_indptr, torch::Tensor& se
            op);
 }
 
+void get_kv_slot_mapping(torch::Tensor& batch_indices, torch::Tensor& positions,
+                         torch::Tensor& kv_indices, torch::Tensor& kv_indptr,
+                         torch::Tensor& slot_mapping, int64_t page_size) {
+  const char* op = "get_kv_slot_mapping";
+  check_i32(batch_indices, batch_indices, op, "batch_indices");
+  check_i32(positions, batch_indices, op, "positions");
+  check_i32(kv_indices, batch_indices, op, "kv_indices");
+  check_i32(kv_indptr, batch_indices, op, "kv_indptr");
+  check_i32(slot_mapping, batch_indices, op, "slot_mapping");
+  const int64_t nnz = batch_indices.numel();
+  TORCH_CHECK(positions.numel() == nnz && slot_mapping.numel() == nnz && page_size > 0, op,
+              ": batch_indices, positions and slot_mapping must hold nnz entries");
+  LaunchScope scope(batch_indices);
+  raise_on(sarathi_get_kv_slot_mapping(batch_indices.data_ptr<int32_t>(),
+                                       positions.data_ptr<int32_t>(),
+                                       kv_indices.data_ptr<int32_t>(),
+                                       kv_indptr.data_ptr<int32_t>(),
+                                       slot_mapping.data_ptr<int32_t>(), nnz, (int)page_size,
+                                       scope.stream),
+           op);
+}
+
 void append_paged_kv_cache(torch::Tensor& append_key, torch::Tensor& append_value,
                            torch::Tensor& batch_indices, torch::Tensor& positions,
                            torch::Tensor& k_cache, torch::Tensor& v_cache,
-                           torch::Tensor& kv_indices, torch::Tensor& kv_indptr) {
+                           torch::Tensor& kv_indices, torch::Tensor& kv_indptr,
+                           c10::optional<torch::Tensor> slot_mapping) {
   const char* op = "append_paged_kv_cache";
   check_gpu(append_key, append_key, op, "append_key");
   check_gpu(append_value, append_key, op, "append_value");
@@ -282,12 +305,18 @@ void append_paged_kv_cache(torch::Tensor& append_key, torch::Tensor& append_valu
   TORCH_CHECK(append_value.size(0) == nnz && batch_indices.numel() == nnz &&
                   positions.numel() == nnz,
               op, ": append_key, append_value, batch_indices and positions disagree on nnz");
+  const int32_t* slots = nullptr;
+  if (slot_mapping.has_value()) {
+    check_i32(*slot_mapping, append_key, op, "slot_mapping");
+    TORCH_CHECK(slot_mapping->numel() == nnz, op, ": slot_mapping must hold nnz entries");
+    slots = slot_mapping->data_ptr<int32_t>();
+  }
   LaunchScope scope(append_key);
   raise_on(sarathi_append_paged_kv_cache(
                append_key.data_ptr(), append_value.data_ptr(), batch_indices.data_ptr<int32_t>(),
                positions.data_ptr<int32_t>(), k_cache.data_ptr(), v_cache.data_ptr(),
-               kv_indices.data_ptr<int32_t>(), kv_indptr.data_ptr<int32_t>(), nnz, (int)g.heads,
-               (int)g.head_size, (int)g.page_size, nnz > 1 ? ks : width, nnz > 1 ? vs : width,
+               kv_indices.data_ptr<int32_t>(), kv_indptr.data_ptr<int32_t>(), slots, nnz,
+               (int)g.heads, (int)g.head_size, (int)g.page_size, nnz > 1 ? ks : width, nnz > 1 ? vs : width,
                g.page_stride, g.entry_stride, dtype_code(append_key, op), scope.stream),
            op);
 }
@@ -299,7 +328,8 @@ void rotary_embedding_append_paged_kv(torch::Tensor& positions, torch::Tensor& q
                                       torch::Tensor& append_positions, torch::Tensor& k_cache,
                                       torch::Tensor& v_cache, torch::Tensor& kv_indices,
                                       torch::Tensor& kv_indptr, int64_t num_append_tokens,
-                                      bool write_key) {
+                                      bool write_key,
+                                      c10::optional<torch::Tensor> slot_mapping) {
   const char* op = "rotary_embedding_append_paged_kv";
   check_gpu(query, query, op, "query");
   check_gpu(key, query, op, "key");
@@ -340,13 +370,20 @@ void rotary_embedding_append_paged_kv(torch::Tensor& positions, torch::Tensor& q
                   batch_indices.numel() >= num_append_tokens &&
                   append_positions.numel() >= num_append_tokens,
               op, ": num_append_tokens must be within num_tokens and the index vectors");
+  const int32_t* slots = nullptr;
+  if (slot_mapping.has_value()) {
+    check_i32(*slot_mapping, query, op, "slot_mapping");
+    TORCH_CHECK(slot_mapping->numel() >= num_append_tokens, op,
+                ": slot_mapping must hold num_append_tokens entries");
+    slots = slot_mapping->data_ptr<int32_t>();
+  }
   LaunchScope scope(query);
   raise_on(sarathi_rotary_embedding_append_paged_kv(
                positions.data_ptr<int64_t>(), query.data_ptr(), key.data_ptr(), value.data_ptr(),
                cos_sin_cache.data_ptr(), batch_indices.data_ptr<int32_t>(),
                append_positions.data_ptr<int32_t>(), k_cache.data_ptr(), v_cache.data_ptr(),
-               kv_indices.data_ptr<int32_t>(), kv_indptr.data_ptr<int32_t>(), T, num_append_tokens,
-               (int)(query.size(1) / head_size), (int)g.heads, (int)head_size, (int)rot_dim,
+               kv_indices.data_ptr<int32_t>(), kv_indptr.data_ptr<int32_t>(), slots, T,
+               num_append_tokens, (int)(query.size(1) / head_size), (int)g.heads, (int)head_size, (int)rot_dim,
                T > 1 ? query.stride(0) : query.size(1), T > 1 ? key.stride(0) : key.size(1),
                T > 1 ? value.stride(0) : value.size(1), (int)g.page_size, g.page_stride,
                g.entry_stride, is_neox ? 1 : 0, write_key ? 1 : 0, dtype_code(query, op),
@@ -527,10 +564,22 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("get_seq_lens", &get_seq_lens, "kv sequence lengths from the page table");
   m.def("get_batch_indices_positions", &get_batch_indices_positions,
         "request index and kv position of every appended token");
+  m.def("get_kv_slot_mapping", &get_kv_slot_mapping,
+        "page * page_size + entry of every appended token");
   m.def("append_paged_kv_cache", &append_paged_kv_cache,
-        "copy key / value rows into their entries of a paged (NHD) KV cache");
+        "copy key / value rows into their entries of a paged (NHD) KV cache",
+        pybind11::arg("append_key"), pybind11::arg("append_value"), pybind11::arg("batch_indices"),
+        pybind11::arg("positions"), pybind11::arg("k_cache"), pybind11::arg("v_cache"),
+        pybind11::arg("kv_indices"), pybind11::arg("kv_indptr"),
+        pybind11::arg("slot_mapping") = pybind11::none());
   m.def("rotary_embedding_append_paged_kv", &rotary_embedding_append_paged_kv,
-        "rotary_embedding fused with append_paged_kv_cache");
+        "rotary_embedding fused with append_paged_kv_cache", pybind11::arg("positions"),
+        pybind11::arg("query"), pybind11::arg("key"), pybind11::arg("value"),
+        pybind11::arg("head_size"), pybind11::arg("cos_sin_cache"), pybind11::arg("is_neox"),
+        pybind11::arg("batch_indices"), pybind11::arg("append_positions"),
+        pybind11::arg("k_cache"), pybind11::arg("v_cache"), pybind11::arg("kv_indices"),
+        pybind11::arg("kv_indptr"), pybind11::arg("num_append_tokens"),
+        pybind11::arg("write_key"), pybind11::arg("slot_mapping") = pybind11::none());
   // moe_ops
   m.def("topk_softmax", &topk_softmax, "softmax over experts + top-k (raw probabilities)");
   m.def("topk_softmax_renorm", &topk_softmax_renorm,

@@ -44,17 +44,29 @@ def get_batch_indices_positions(append_indptr: torch.Tensor, seq_lens: torch.Ten
     return batch_indices, positions
 
 
+def get_kv_slot_mapping(batch_indices: torch.Tensor, positions: torch.Tensor,
+                        kv_indices: torch.Tensor, kv_indptr: torch.Tensor,
+                        page_size: int) -> torch.Tensor:
+    """``page * page_size + entry`` of every appended token.  The page table of a batch is the
+    same for all layers: compute this once per batch and pass it as ``slot_mapping`` to the append
+    ops, which then resolve a token's destination with one index load instead of three."""
+    slot_mapping = torch.empty_like(batch_indices)
+    _C.get_kv_slot_mapping(batch_indices, positions, kv_indices, kv_indptr, slot_mapping, page_size)
+    return slot_mapping
+
+
 def append_paged_kv_cache(append_key: torch.Tensor, append_value: torch.Tensor,
                           batch_indices: torch.Tensor, positions: torch.Tensor,
                           paged_kv_cache: PagedCache, kv_indices: torch.Tensor,
                           kv_indptr: torch.Tensor, kv_last_page_len: Optional[torch.Tensor] = None,
-                          kv_layout: str = "NHD") -> None:
+                          kv_layout: str = "NHD",
+                          slot_mapping: Optional[torch.Tensor] = None) -> None:
     """Copy ``append_key`` / ``append_value`` ``[nnz, num_kv_heads, head_size]`` into the cache.
     ``kv_last_page_len`` is accepted for signature compatibility; the destination of a token
     follows from ``positions`` alone."""
     k_cache, v_cache = _split_cache(paged_kv_cache, kv_layout)
     _C.append_paged_kv_cache(append_key, append_value, batch_indices, positions, k_cache, v_cache,
-                             kv_indices, kv_indptr)
+                             kv_indices, kv_indptr, slot_mapping)
 
 
 def rotary_embedding_append_paged_kv(positions: torch.Tensor, query: torch.Tensor,
@@ -64,7 +76,8 @@ def rotary_embedding_append_paged_kv(positions: torch.Tensor, query: torch.Tenso
                                      paged_kv_cache: PagedCache, kv_indices: torch.Tensor,
                                      kv_indptr: torch.Tensor,
                                      num_append_tokens: Optional[int] = None,
-                                     write_key: bool = False, kv_layout: str = "NHD") -> None:
+                                     write_key: bool = False, kv_layout: str = "NHD",
+                                     slot_mapping: Optional[torch.Tensor] = None) -> None:
     """``pos_encoding_ops.rotary_embedding(positions, query, key, ...)`` followed by
     ``append_paged_kv_cache(key[:n], value[:n], ...)`` in one launch (n = ``num_append_tokens``,
     default all tokens).  ``query`` is rotated in place; the rotated keys go to the cache and, only
@@ -73,8 +86,8 @@ def rotary_embedding_append_paged_kv(positions: torch.Tensor, query: torch.Tenso
     n = positions.shape[0] if num_append_tokens is None else int(num_append_tokens)
     _C.rotary_embedding_append_paged_kv(positions, query, key, value, head_size, cos_sin_cache,
                                         is_neox, batch_indices, append_positions, k_cache, v_cache,
-                                        kv_indices, kv_indptr, n, write_key)
+                                        kv_indices, kv_indptr, n, write_key, slot_mapping)
 
 
-__all__ = ["get_seq_lens", "get_batch_indices_positions", "append_paged_kv_cache",
+__all__ = ["get_seq_lens", "get_batch_indices_positions", "get_kv_slot_mapping", "append_paged_kv_cache",
            "rotary_embedding_append_paged_kv"]

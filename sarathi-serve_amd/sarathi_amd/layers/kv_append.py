@@ -34,6 +34,7 @@ class AppendMetadata:
     append_kv_last_page_len: torch.Tensor   # [requests]
     append_batch_indices: torch.Tensor      # [num_total_tokens]
     append_positions: torch.Tensor          # [num_total_tokens]
+    slot_mapping: torch.Tensor              # [num_total_tokens] page * block_size + entry
     num_prefill_tokens: int
     num_total_tokens: int
 
@@ -71,5 +72,7 @@ def build_append_metadata(seqs: Sequence[SequenceSlice], block_size: int,
     seq_lens = kv_cache_ops.get_seq_lens(m_indptr, m_last, block_size)
     batch_indices, positions = kv_cache_ops.get_batch_indices_positions(m_qo, seq_lens,
                                                                         num_total_tokens)
-    return AppendMetadata(m_qo, m_idx, m_indptr, m_last, batch_indices, positions,
+    slot_mapping = kv_cache_ops.get_kv_slot_mapping(batch_indices, positions, m_idx, m_indptr,
+                                                    block_size)
+    return AppendMetadata(m_qo, m_idx, m_indptr, m_last, batch_indices, positions, slot_mapping,
                           num_prefill_tokens, num_total_tokens)

@@ -146,11 +146,14 @@ def test_kv_cache_and_gemm_argument_validation_without_gpu(lib):
 
     def append(**kw):
         return lib.sarathi_append_paged_kv_cache(
-            kw.get("key", p), p, p, p, p, kw.get("vc", p), p, p, i64(kw.get("nnz", 1)), ci(2),
+            kw.get("key", p), p, kw.get("bi", p), p, p, kw.get("vc", p), p, p, kw.get("slots", null),
+            i64(kw.get("nnz", 1)), ci(2),
             ci(8), ci(kw.get("page", 4)), i64(kw.get("ks", 16)), i64(16),
             i64(kw.get("ps", 64)), i64(kw.get("es", 16)), ci(kw.get("dt", 2)), null)
     assert append(key=null) == INVALID
     assert append(vc=null) == INVALID
+    assert append(bi=null) == INVALID     # neither index arrays nor a slot mapping
+    assert append(bi=null, slots=p, nnz=0) == OK
     assert append(ks=8) == INVALID        # key rows narrower than heads * head_size
     assert append(es=8) == INVALID        # cache entries narrower than a row
     assert append(ps=32) == INVALID       # page stride < page_size * entry stride
@@ -163,10 +166,13 @@ def test_kv_cache_and_gemm_argument_validation_without_gpu(lib):
     assert lib.sarathi_get_seq_lens(p, p, p, i64(0), ci(4), null) == OK
     assert lib.sarathi_get_batch_indices_positions(p, p, null, p, i64(1), i64(1), null) == INVALID
     assert lib.sarathi_get_batch_indices_positions(p, p, p, p, i64(0), i64(0), null) == OK
+    assert lib.sarathi_get_kv_slot_mapping(p, p, p, p, null, i64(1), ci(4), null) == INVALID
+    assert lib.sarathi_get_kv_slot_mapping(p, p, p, p, p, i64(0), ci(4), null) == OK
 
     def fused(**kw):
         return lib.sarathi_rotary_embedding_append_paged_kv(
-            kw.get("pos", p), p, p, kw.get("value", p), p, p, p, p, p, p, p, i64(kw.get("T", 1)),
+            kw.get("pos", p), p, p, kw.get("value", p), p, p, p, p, p, p, p, null,
+            i64(kw.get("T", 1)),
             i64(kw.get("n", 1)), ci(2), ci(1), ci(16), ci(kw.get("rot", 16)), i64(32),
             i64(kw.get("ks", 16)), i64(16), ci(4), i64(64), i64(16), ci(1), ci(0),
             ci(kw.get("dt", 2)), null)

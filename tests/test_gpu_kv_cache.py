@@ -94,6 +94,15 @@ def test_append_matches_oracle_bitwise(ops, dev, dtype, page_size, before, new, 
     ops.kv_cache_ops.append_paged_kv_cache(qkv[:, 2 * w:3 * w], qkv[:, 3 * w:], t(b), t(pos),
                                            (kc, vc), t(kv_indices), t(kv_indptr))
     assert np.array_equal(_bits(kc.cpu()), want[:, 0]) and np.array_equal(_bits(vc.cpu()), want[:, 1])
+    # precomputed slot mapping: same bytes
+    slots = ops.kv_cache_ops.get_kv_slot_mapping(t(b), t(pos), t(kv_indices), t(kv_indptr), page_size)
+    want_slots = [int(kv_indices[kv_indptr[bi] + p // page_size]) * page_size + p % page_size
+                  for bi, p in zip(b.tolist(), pos.tolist())]
+    assert slots.cpu().tolist() == want_slots
+    got2 = cache.to(dev)
+    ops.kv_cache_ops.append_paged_kv_cache(k.to(dev), v.to(dev), t(b), t(pos), got2, t(kv_indices),
+                                           t(kv_indptr), slot_mapping=slots)
+    assert np.array_equal(_bits(got2.cpu()), want)
 
 
 def _rope_then_append(positions, q, k, v, head_size, table, is_neox, b, pos, cache, kv_indices,
@@ -145,6 +154,15 @@ def test_fused_rope_append_equals_separate_ops(ops, dev, dtype, is_neox, nq, nkv
         positions.to(dev), q, k, v, head_size, table.to(dev), is_neox, t(b), t(pos), got_cache,
         t(kv_indices), t(kv_indptr), num_append_tokens=n, write_key=write_key)
     assert np.array_equal(_bits(got_cache.cpu()), _bits(want_cache))
+    # the same call with the destinations resolved beforehand
+    slots = ops.kv_cache_ops.get_kv_slot_mapping(t(b), t(pos), t(kv_indices), t(kv_indptr), page_size)
+    dq2 = qkv.to(dev)
+    q2, k2, v2 = dq2.split([nq * head_size, nkv * head_size, nkv * head_size], dim=-1)
+    got_cache2 = cache.to(dev)
+    ops.kv_cache_ops.rotary_embedding_append_paged_kv(
+        positions.to(dev), q2, k2, v2, head_size, table.to(dev), is_neox, t(b), t(pos), got_cache2,
+        t(kv_indices), t(kv_indptr), num_append_tokens=n, write_key=write_key, slot_mapping=slots)
+    assert torch.equal(got_cache2, got_cache) and torch.equal(dq2, dq)
     out = dq.cpu()
     oq, ok, ov = out.split([nq * head_size, nkv * head_size, nkv * head_size], dim=-1)
     assert np.array_equal(_bits(oq), _bits(rq))
