@@ -40,6 +40,8 @@ HIP_FLAGS = [
     "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wall", "-Wno-unused-command-line-argument",
 ]
+# extra hipcc flags for tuning builds, e.g. -DSARATHI_KV_STORE_POLICY=18
+HIP_FLAGS += os.environ.get("SARATHI_HIPCC_EXTRA_FLAGS", "").split()
 
 
 def _run(cmd, verbose):

@@ -27,7 +27,7 @@ __global__ __launch_bounds__(64) void kv_append_seg_kernel(
                     tok * (is_k ? k_stride_bytes : v_stride_bytes);
   const u32x4 v = buf_load16<kStreamLoad>(make_rsrc(src, row_bytes), off);
   char* dst = reinterpret_cast<char*>(is_k ? d.k_cache : d.v_cache) + kv_entry_offset(d, tok);
-  buf_store16<kCached>(make_rsrc(dst, row_bytes), off, v);  // pieces past the row are dropped
+  buf_store16<kKvStore>(make_rsrc(dst, row_bytes), off, v);  // pieces past the row are dropped
 }
 
 // Any alignment: one workgroup per token, 2-byte units (every supported dtype is a multiple).

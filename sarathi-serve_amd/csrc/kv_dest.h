@@ -15,6 +15,12 @@
 
 namespace sarathi_hip {
 
+// Cache policy of the stores into cache entries (overridable for tuning runs).
+#ifndef SARATHI_KV_STORE_POLICY
+#define SARATHI_KV_STORE_POLICY 0
+#endif
+constexpr int kKvStore = SARATHI_KV_STORE_POLICY;
+
 struct KvDest {
   const int32_t* batch_indices;  // [nnz]
   const int32_t* positions;      // [nnz] index of the token inside its request's kv sequence

@@ -226,7 +226,7 @@ __global__ __launch_bounds__(64) void rope_append_seg_kernel(
     const char* src = reinterpret_cast<const char*>(value) + tok * (int64_t)v_stride_bytes;
     const u32x4 v = buf_load16<kStreamLoad>(make_rsrc(src, kv_row_bytes), off);
     char* dst = reinterpret_cast<char*>(d.v_cache) + kv_entry_offset(d, tok);
-    buf_store16<kCached>(make_rsrc(dst, kv_row_bytes), off, v);
+    buf_store16<kKvStore>(make_rsrc(dst, kv_row_bytes), off, v);
     return;
   }
 
@@ -283,8 +283,8 @@ __global__ __launch_bounds__(64) void rope_append_seg_kernel(
       buf_store16<kStreamStore>(rd, xoff + embed_bytes, py);
     }
     if (to_cache) {
-      buf_store16<kCached>(rk, xoff, px);
-      buf_store16<kCached>(rk, xoff + embed_bytes, py);
+      buf_store16<kKvStore>(rk, xoff, px);
+      buf_store16<kKvStore>(rk, xoff + embed_bytes, py);
     }
   } else {
     Vec<DT> o;
@@ -296,7 +296,7 @@ __global__ __launch_bounds__(64) void rope_append_seg_kernel(
     }
     const u32x4 po = o.pack();
     if (in_place) buf_store16<kStreamStore>(rd, xoff, po);
-    if (to_cache) buf_store16<kCached>(rk, xoff, po);
+    if (to_cache) buf_store16<kKvStore>(rk, xoff, po);
   }
 }
 
