@@ -65,6 +65,8 @@ BYTES["topk_softmax"] = MOE_T * MOE_E * 4 + 3 * MOE_T * MOE_K * 4
 _moe_sorted = MOE_T * MOE_K + MOE_E * (MOE_B - 1)
 BYTES["moe_align_block_size"] = MOE_T * MOE_K * 4 + _moe_sorted * 4 + 4 * (
     (_moe_sorted + MOE_B - 1) // MOE_B) + 4
+# both in one launch: the ids are written once and re-read from L2
+BYTES["fused_topk_align"] = BYTES["topk_softmax"] + BYTES["moe_align_block_size"]
 
 
 # HBM bytes per silu_and_mul launch at this shape as measured with rocprofv3 --pmc FETCH_SIZE and
@@ -254,6 +256,8 @@ def main():
         "topk_softmax": ([None], lambda a: MOE.topk_softmax(tw, ti, ts, gating)),
         "moe_align_block_size": ([None], lambda a: MOE.moe_align_block_size_filled(
             ti, MOE_E, MOE_B, sorted_ids, expert_ids, post_pad)),
+        "fused_topk_align": ([None], lambda a: MOE.fused_topk_align(
+            tw, ti, ts, gating, True, MOE_B, sorted_ids, expert_ids, post_pad, True)),
     }
 
     def time_op(fn, args, reps):
@@ -272,7 +276,7 @@ def main():
     per_op = {}
     for name, (args_ring, fn) in ops_table.items():
         row = {"bytes": BYTES[name]}
-        latency_bound = name in ("topk_softmax", "moe_align_block_size")
+        latency_bound = name in ("topk_softmax", "moe_align_block_size", "fused_topk_align")
         for label in ("cold", "warm"):
             if latency_bound and label == "cold":
                 continue   # 0.07-0.2 MB working sets: launch-latency-bound, one (warm) figure

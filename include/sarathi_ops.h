@@ -162,6 +162,24 @@ int sarathi_moe_align_block_size(const void* topk_ids, int id_dtype, int64_t num
 int64_t sarathi_moe_align_workspace_bytes(int64_t numel, int num_experts);
 
 /*
+ * New entry: sarathi_topk_softmax followed by sarathi_moe_align_block_size (on the int32 ids it
+ * just produced) in ONE launch, for the reference's per-layer sequence
+ * fused_topk -> moe_align_block_size (sarathi/model_executor/layers/fused_moe/fused_moe.py:346-373
+ * and :151-204).  Outputs are bit-identical to the two separate calls.  `counter` is one uint32
+ * of device memory that is zero before the first call; the call leaves it zero again.  Calls
+ * that share a counter must not overlap (use one counter per stream).  With counter = NULL, with
+ * an expert count that is not a power of two up to 256, or with more than 16384 ids, the two
+ * stand-alone kernels are launched instead.
+ */
+int sarathi_fused_topk_align(float* topk_weights, int32_t* topk_indices,
+                             int32_t* token_expert_indices, const float* gating_output,
+                             int64_t num_tokens, int num_experts, int topk, int renormalize,
+                             int block_size, int32_t* sorted_token_ids, int64_t sorted_len,
+                             int32_t* expert_ids, int64_t expert_ids_len,
+                             int32_t* num_tokens_post_pad, int fill_pad, uint32_t* counter,
+                             void* stream);
+
+/*
  * Grouped expert GEMM that consumes moe_align_block_size's outputs; replaces the
  * Triton kernel launched by invoke_fused_moe_kernel
  * (sarathi/model_executor/layers/fused_moe/fused_moe.py:15-148, :207-260).

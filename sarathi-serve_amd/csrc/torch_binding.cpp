@@ -13,6 +13,10 @@
 #include <hip/hip_runtime_api.h>
 #include <torch/extension.h>
 
+#include <map>
+#include <mutex>
+#include <utility>
+
 #include "../../include/sarathi_ops.h"
 
 namespace {
@@ -485,6 +489,66 @@ void moe_align_block_size_filled(torch::Tensor topk_ids, int64_t num_experts, in
                  num_tokens_post_pad, true, "moe_align_block_size_filled");
 }
 
+// One zeroed uint32 per (device, stream): the completion counter of the fused routing kernel.
+// Allocated on first use and kept for the life of the process.
+uint32_t* routing_counter(int dev, void* stream) {
+  static std::mutex mu;
+  static std::map<std::pair<int, void*>, torch::Tensor> counters;
+  std::lock_guard<std::mutex> lock(mu);
+  auto key = std::make_pair(dev, stream);
+  auto it = counters.find(key);
+  if (it == counters.end()) {
+    auto t = torch::zeros({1}, torch::TensorOptions().dtype(torch::kInt32).device(torch::kCUDA, dev));
+    it = counters.emplace(key, t).first;
+  }
+  return reinterpret_cast<uint32_t*>(it->second.data_ptr<int32_t>());
+}
+
+// fused_topk + moe_align_block_size of fused_moe.py:346-373 / :151-204 in one launch
+void fused_topk_align(torch::Tensor& topk_weights, torch::Tensor& topk_indices,
+                      torch::Tensor& token_expert_indices, torch::Tensor& gating_output,
+                      bool renormalize, int64_t block_size, torch::Tensor& sorted_token_ids,
+                      torch::Tensor& experts_ids, torch::Tensor& num_tokens_post_pad,
+                      bool fill_pad) {
+  const char* op = "fused_topk_align";
+  check_gpu(gating_output, gating_output, op, "gating_output");
+  check_gpu(topk_weights, gating_output, op, "topk_weights");
+  check_gpu(topk_indices, gating_output, op, "topk_indices");
+  check_gpu(token_expert_indices, gating_output, op, "token_expert_indices");
+  check_gpu(sorted_token_ids, gating_output, op, "sorted_token_ids");
+  check_gpu(experts_ids, gating_output, op, "experts_ids");
+  check_gpu(num_tokens_post_pad, gating_output, op, "num_tokens_post_pad");
+  TORCH_CHECK(gating_output.scalar_type() == at::ScalarType::Float &&
+                  topk_weights.scalar_type() == at::ScalarType::Float,
+              op, ": gating_output and topk_weights must be float32");
+  TORCH_CHECK(topk_indices.scalar_type() == at::ScalarType::Int &&
+                  token_expert_indices.scalar_type() == at::ScalarType::Int &&
+                  sorted_token_ids.scalar_type() == at::ScalarType::Int &&
+                  experts_ids.scalar_type() == at::ScalarType::Int &&
+                  num_tokens_post_pad.scalar_type() == at::ScalarType::Int,
+              op, ": index tensors must be int32");
+  TORCH_CHECK(gating_output.dim() == 2 && gating_output.is_contiguous() &&
+                  topk_weights.is_contiguous() && topk_indices.is_contiguous() &&
+                  token_expert_indices.is_contiguous() && sorted_token_ids.is_contiguous() &&
+                  experts_ids.is_contiguous() && num_tokens_post_pad.numel() >= 1,
+              op, ": tensors must be contiguous");
+  const int64_t T = gating_output.size(0), E = gating_output.size(1);
+  TORCH_CHECK(topk_weights.dim() == 2 && topk_weights.size(0) == T, op,
+              ": topk_weights must be [num_tokens, topk]");
+  const int64_t k = topk_weights.size(1);
+  TORCH_CHECK(topk_indices.numel() == T * k && token_expert_indices.numel() == T * k, op,
+              ": topk outputs must be [num_tokens, topk]");
+  LaunchScope scope(gating_output);
+  raise_on(sarathi_fused_topk_align(
+               topk_weights.data_ptr<float>(), topk_indices.data_ptr<int32_t>(),
+               token_expert_indices.data_ptr<int32_t>(), gating_output.data_ptr<float>(), T, (int)E,
+               (int)k, renormalize ? 1 : 0, (int)block_size, sorted_token_ids.data_ptr<int32_t>(),
+               sorted_token_ids.numel(), experts_ids.data_ptr<int32_t>(), experts_ids.numel(),
+               num_tokens_post_pad.data_ptr<int32_t>(), fill_pad ? 1 : 0,
+               routing_counter(scope.dev, scope.stream), scope.stream),
+           op);
+}
+
 // A [tokens, K], B [E, N, K], C [tokens, topk, N] (or any tensor whose rows of N elements are
 // addressed by slot = token * topk + j), as invoke_fused_moe_kernel passes them.  With
 // b_packed, B is the re-tiled weight tensor [E, ceil(N/32), K/16, 2, 32, 8] and `n` its logical
@@ -588,6 +652,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "stable sort of token ids by expert, runs padded to block_size");
   m.def("moe_align_block_size_filled", &moe_align_block_size_filled,
         "moe_align_block_size that also writes the padding value into unused slots");
+  m.def("fused_topk_align", &fused_topk_align,
+        "topk_softmax (+ optional renormalisation) and moe_align_block_size in one launch");
   m.def("moe_grouped_gemm", &moe_grouped_gemm,
         "C[slot] = A[slot / top_k] @ B[expert(slot)]^T over moe_align_block_size's layout",
         pybind11::arg("a"), pybind11::arg("b"), pybind11::arg("c"), pybind11::arg("topk_weights"),

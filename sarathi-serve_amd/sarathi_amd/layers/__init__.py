@@ -6,13 +6,13 @@ from .activation import FastGELU, NewGELU, SiluAndMul, get_act_fn
 from .fused_moe import (PackedExpertWeights, fused_experts, fused_moe, invoke_fused_moe_kernel,
                         pack_expert_weights)
 from .kv_append import AppendMetadata, SequenceSlice, build_append_metadata
-from .moe_routing import fused_topk, moe_align_block_size
+from .moe_routing import fused_topk, fused_topk_and_align, moe_align_block_size
 from .norm import RMSNorm
 from .rotary import (DynamicNTKScalingRotaryEmbedding, LinearScalingRotaryEmbedding,
                      RotaryEmbedding, YaRNScalingRotaryEmbedding, get_rope)
 
 __all__ = ["RMSNorm", "SiluAndMul", "NewGELU", "FastGELU", "get_act_fn", "RotaryEmbedding",
            "LinearScalingRotaryEmbedding", "DynamicNTKScalingRotaryEmbedding",
-           "YaRNScalingRotaryEmbedding", "get_rope", "fused_topk", "moe_align_block_size",
+           "YaRNScalingRotaryEmbedding", "get_rope", "fused_topk", "fused_topk_and_align", "moe_align_block_size",
            "invoke_fused_moe_kernel", "fused_experts", "fused_moe", "pack_expert_weights",
            "PackedExpertWeights", "SequenceSlice", "AppendMetadata", "build_append_metadata"]

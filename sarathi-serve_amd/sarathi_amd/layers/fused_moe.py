@@ -12,7 +12,7 @@ from typing import Any, Dict, Optional
 import torch
 
 from .. import activation_ops, moe_ops
-from .moe_routing import fused_topk, moe_align_block_size
+from .moe_routing import fused_topk, fused_topk_and_align, moe_align_block_size
 
 _BLOCK_SIZES = (32, 64, 128, 256)
 
@@ -46,6 +46,12 @@ def pack_expert_weights(w: torch.Tensor) -> PackedExpertWeights:
     return PackedExpertWeights(tiles, (E, N, K))
 
 
+# (token, k) slots up to which fused_moe routes with the one-launch kernel (it covers 16384).
+# Off by default: measured on MI355X at 4096 tokens x top-2 of 8 experts the single launch takes
+# 13.7 us against 12.8 us for the two kernels back to back (the sorting workgroup has to read the
+# ids through device-coherent loads, which costs what the saved launch gains); it only pays when
+# the host, not the GPU, is the bottleneck of the launch sequence.
+FUSED_ROUTING_MAX_SLOTS = 0
 CHUNK_SIZE = 64 * 1024     # tokens per pass, as in the reference (fused_moe.py:437)
 
 
@@ -83,7 +89,9 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
                   override_config: Optional[Dict[str, Any]] = None,
                   w1_scale: Optional[torch.Tensor] = None, w2_scale: Optional[torch.Tensor] = None,
                   a1_scale: Optional[torch.Tensor] = None,
-                  a2_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  a2_scale: Optional[torch.Tensor] = None, _alignment=None) -> torch.Tensor:
+    """``_alignment``: (sorted_token_ids, expert_ids, num_tokens_post_padded, block_size) already
+    computed for the whole batch by the fused routing launch (single-chunk batches only)."""
     assert hidden_states.shape[1] == w1.shape[2], "Hidden size mismatch"
     assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
     assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
@@ -113,7 +121,11 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
         cur_ids, cur_w = topk_ids[begin:end], topk_weights[begin:end]
         config = override_config or get_default_config(n, E, w2.shape[1], K, topk)
         c1, c2, c3 = cache1[:n], cache2[:n * topk], cache3[:n]
-        sorted_ids, expert_ids, post_padded = moe_align_block_size(cur_ids, config["BLOCK_SIZE_M"], E)
+        if _alignment is not None and n == num_tokens and _alignment[3] == config["BLOCK_SIZE_M"]:
+            sorted_ids, expert_ids, post_padded = _alignment[:3]
+        else:
+            sorted_ids, expert_ids, post_padded = moe_align_block_size(
+                cur_ids, config["BLOCK_SIZE_M"], E)
         invoke_fused_moe_kernel(cur_hidden, w1, c1, None, None, cur_w, cur_ids, sorted_ids,
                                 expert_ids, post_padded, False, topk, config)
         activation_ops.silu_and_mul(c2, c1.view(-1, N))
@@ -135,7 +147,18 @@ def fused_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
     assert gating_output.shape[1] == w1.shape[0], "Number of experts mismatch"
     if use_grouped_topk:
         raise NotImplementedError("grouped_topk (DeepSeek-V2 routing) is not part of this library")
-    topk_weights, topk_ids = fused_topk(hidden_states, gating_output, topk, renormalize)
+    num_tokens, E = gating_output.shape
+    alignment = None
+    if 0 < num_tokens * topk <= FUSED_ROUTING_MAX_SLOTS:
+        # small batches are launch-latency bound: routing and slot sort in one launch
+        config = override_config or get_default_config(num_tokens, E, w2.shape[1],
+                                                       hidden_states.shape[1], topk)
+        block_m = config["BLOCK_SIZE_M"]
+        topk_weights, topk_ids, sorted_ids, expert_ids, post_padded = fused_topk_and_align(
+            hidden_states, gating_output, topk, renormalize, block_m)
+        alignment = (sorted_ids, expert_ids, post_padded, block_m)
+    else:
+        topk_weights, topk_ids = fused_topk(hidden_states, gating_output, topk, renormalize)
     return fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, inplace=inplace,
                          override_config=override_config, w1_scale=w1_scale, w2_scale=w2_scale,
-                         a1_scale=a1_scale, a2_scale=a2_scale)
+                         a1_scale=a1_scale, a2_scale=a2_scale, _alignment=alignment)

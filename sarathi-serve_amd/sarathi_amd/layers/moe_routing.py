@@ -39,3 +39,27 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int,
     moe_ops.moe_align_block_size_filled(topk_ids.contiguous(), num_experts, block_size, sorted_ids,
                                         expert_ids, num_tokens_post_pad)
     return sorted_ids, expert_ids, num_tokens_post_pad
+
+
+def fused_topk_and_align(hidden_states: torch.Tensor, gating_output: torch.Tensor, topk: int,
+                         renormalize: bool, block_size: int):
+    """``fused_topk`` followed by ``moe_align_block_size`` as ONE kernel launch (up to 16384
+    (token, k) slots and a power-of-two expert count up to 256; other shapes run the two kernels).
+    Returns (topk_weights, topk_ids, sorted_token_ids, expert_ids, num_tokens_post_padded), the
+    same tensors the two separate calls return."""
+    assert hidden_states.shape[0] == gating_output.shape[0], "Number of tokens mismatch"
+    M, E = gating_output.shape
+    dev = hidden_states.device
+    topk_weights = torch.empty((M, topk), dtype=torch.float32, device=dev)
+    topk_ids = torch.empty((M, topk), dtype=torch.int32, device=dev)
+    token_expert_indices = torch.empty((M, topk), dtype=torch.int32, device=dev)
+    max_padded = M * topk + E * (block_size - 1)
+    sorted_ids = torch.empty((max_padded,), dtype=torch.int32, device=dev)
+    expert_ids = torch.empty(((max_padded + block_size - 1) // block_size,), dtype=torch.int32,
+                             device=dev)
+    num_tokens_post_pad = torch.empty((1,), dtype=torch.int32, device=dev)
+    logits = gating_output if gating_output.dtype == torch.float32 else gating_output.float()
+    moe_ops.fused_topk_align(topk_weights, topk_ids, token_expert_indices, logits.contiguous(),
+                             renormalize, block_size, sorted_ids, expert_ids, num_tokens_post_pad,
+                             True)
+    return topk_weights, topk_ids, sorted_ids, expert_ids, num_tokens_post_pad

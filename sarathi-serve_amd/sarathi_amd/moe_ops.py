@@ -14,6 +14,10 @@ moe_align_block_size_filled = _C.moe_align_block_size_filled
 # grouped expert GEMM over moe_align_block_size's layout: what the reference launches as a Triton
 # kernel from invoke_fused_moe_kernel (layers/fused_moe/fused_moe.py:207-260)
 moe_grouped_gemm = _C.moe_grouped_gemm
+# fused_topk_align(topk_weights, topk_ids, token_expert_indices, gating_output, renormalize,
+#                  block_size, sorted_token_ids, experts_ids, num_tokens_post_pad, fill_pad):
+# topk_softmax(_renorm) and moe_align_block_size(_filled) in one launch, same outputs
+fused_topk_align = _C.fused_topk_align
 
 __all__ = ["topk_softmax", "moe_align_block_size", "topk_softmax_renorm",
-           "moe_align_block_size_filled", "moe_grouped_gemm"]
+           "moe_align_block_size_filled", "moe_grouped_gemm", "fused_topk_align"]

@@ -121,3 +121,19 @@ def test_fused_moe_forward(ops, dev, T, E, k, H, I, renorm):
     out = layers.fused_moe(xd, w1.to(dev), w2.to(dev), gating.to(dev), k, renorm, inplace=True)
     assert out.data_ptr() == xd.data_ptr()
     _close(xd, want, "fused_moe inplace")
+
+
+def test_fused_moe_with_one_launch_routing(ops, dev, monkeypatch):
+    """fused_moe with the routing + slot sort done by the single fused launch: same bits."""
+    from sarathi_amd import layers
+    from sarathi_amd.layers import fused_moe as fm
+    T, E, k, H, I = 300, 8, 2, 256, 512
+    g = gen(21)
+    x = randn((T, H), g, std=1.0).to(dev)
+    w1 = randn((E, 2 * I, H), g, std=H ** -0.5).to(dev)
+    w2 = randn((E, H, I), g, std=I ** -0.5).to(dev)
+    gating = torch.randn((T, E), generator=g, dtype=torch.float32).to(dev)
+    want = layers.fused_moe(x, w1, w2, gating, k, True)
+    monkeypatch.setattr(fm, "FUSED_ROUTING_MAX_SLOTS", 16384)
+    got = layers.fused_moe(x, w1, w2, gating, k, True)
+    assert torch.equal(got, want)

@@ -224,3 +224,73 @@ def test_moe_align_workspace_is_optional(ops, dev):
         assert rc == 0
         torch.cuda.synchronize()
         _check_align((gs.cpu(), ge.cpu(), gp.cpu()), (ws, we, wp), B)
+
+
+# ---- topk_softmax + moe_align_block_size in one launch -------------------------------------------
+
+def _separate(ops, dev, gating, k, renorm, E, B):
+    T = gating.shape[0]
+    w = torch.empty((T, k), dtype=torch.float32, device=dev)
+    idx = torch.empty((T, k), dtype=torch.int32, device=dev)
+    src = torch.empty((T, k), dtype=torch.int32, device=dev)
+    (ops.moe_ops.topk_softmax_renorm if renorm else ops.moe_ops.topk_softmax)(w, idx, src, gating)
+    n = T * k + E * (B - 1)
+    s = torch.full((n,), -5, dtype=torch.int32, device=dev)
+    e = torch.full(((n + B - 1) // B,), -5, dtype=torch.int32, device=dev)
+    p = torch.full((1,), -5, dtype=torch.int32, device=dev)
+    ops.moe_ops.moe_align_block_size_filled(idx, E, B, s, e, p)
+    return w, idx, src, s, e, p
+
+
+@pytest.mark.parametrize("T,E,k,B,renorm", [
+    (4096, 8, 2, 64, True),        # Mixtral routing of the benchmark batch
+    (4096, 8, 2, 128, False),
+    (1, 8, 2, 16, True),           # a single token: one workgroup, which is also the last one
+    (17, 2, 1, 4, False),
+    (515, 64, 6, 32, True),        # several workgroups, ragged last row block
+    (2048, 256, 8, 16, False),     # 16384 slots: the largest fused case
+    (300, 16, 4, 64, True),
+    (2049, 256, 8, 16, True),      # one slot too many: two launches, same results
+    (700, 60, 4, 32, False),       # expert count not a power of two: two launches
+])
+def test_fused_topk_align_equals_separate_ops(ops, dev, T, E, k, B, renorm):
+    """Several calls on the same output buffers with different logits: the completion counter must
+    be back at zero after every call, and the sorting workgroup must see the ids of THIS call,
+    not lines cached from the previous one."""
+    n = T * k + E * (B - 1)
+    w = torch.empty((T, k), dtype=torch.float32, device=dev)
+    idx = torch.empty((T, k), dtype=torch.int32, device=dev)
+    src = torch.empty((T, k), dtype=torch.int32, device=dev)
+    s = torch.empty((n,), dtype=torch.int32, device=dev)
+    e = torch.empty(((n + B - 1) // B,), dtype=torch.int32, device=dev)
+    p = torch.empty((1,), dtype=torch.int32, device=dev)
+    for rep in range(4):
+        gating = torch.randn((T, E), generator=gen(T + E + 1000 * rep), dtype=torch.float32).to(dev)
+        want = _separate(ops, dev, gating, k, renorm, E, B)
+        s.fill_(-5)
+        e.fill_(-5)
+        ops.moe_ops.fused_topk_align(w, idx, src, gating, renorm, B, s, e, p, True)
+        for got, exp, name in zip((w, idx, src, s, e, p), want,
+                                  ("weights", "ids", "source", "sorted", "expert_ids", "post_pad")):
+            assert torch.equal(got, exp), "%s differ on call %d" % (name, rep)
+
+
+def test_fused_topk_align_against_oracle(ops, dev):
+    """The one-launch path against the CPU oracle directly (not only against the other kernels)."""
+    T, E, k, B = 1000, 8, 2, 64
+    gating = torch.randn((T, E), generator=gen(77), dtype=torch.float32)
+    _assert_separated(gating, k)
+    ww, wi, ws = _topk_oracle(gating, k)
+    n = T * k + E * (B - 1)
+    os_ = torch.full((n,), T * k, dtype=torch.int32)
+    oe = torch.zeros(((n + B - 1) // B,), dtype=torch.int32)
+    op = torch.zeros((1,), dtype=torch.int32)
+    c_oracle.moe_align_block_size(wi, E, B, os_, oe, op)
+    from sarathi_amd import layers
+    w, idx, s, e, p = layers.fused_topk_and_align(torch.empty((T, 4), device=dev), gating.to(dev), k,
+                                                  False, B)
+    assert torch.equal(idx.cpu(), wi) and torch.allclose(w.cpu(), ww, rtol=0, atol=1e-6)
+    assert int(p.item()) == int(op.item())
+    assert torch.equal(s.cpu(), os_)
+    nb = int(op.item()) // B
+    assert torch.equal(e.cpu()[:nb], oe[:nb])
