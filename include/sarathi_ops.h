@@ -162,6 +162,21 @@ int sarathi_moe_align_block_size(const void* topk_ids, int id_dtype, int64_t num
 int64_t sarathi_moe_align_workspace_bytes(int64_t numel, int num_experts);
 
 /*
+ * Replaces grouped_topk(hidden_states, gating_output, topk, renormalize, num_expert_group,
+ * topk_group), which the reference writes with tensor ops
+ * (sarathi/model_executor/layers/fused_moe/fused_moe.py:377-408): softmax over the experts; the
+ * experts form num_expert_group consecutive groups of equal size; the topk_group groups with the
+ * largest member probability are kept and every other expert's probability is replaced by 0;
+ * then the top-k of the result, optionally divided by their sum.  The reference's torch.topk
+ * (sorted=False) leaves the output order and the choice among equal values unspecified; here
+ * outputs are in descending order and equal values resolve to the lower index.
+ * num_experts <= SARATHI_MOE_MAX_EXPERTS, num_expert_group <= 64 and a divisor of num_experts.
+ */
+int sarathi_grouped_topk(float* topk_weights, int32_t* topk_indices, const float* gating_output,
+                         int64_t num_tokens, int num_experts, int topk, int num_expert_group,
+                         int topk_group, int renormalize, void* stream);
+
+/*
  * New entry: sarathi_topk_softmax followed by sarathi_moe_align_block_size (on the int32 ids it
  * just produced) in ONE launch, for the reference's per-layer sequence
  * fused_topk -> moe_align_block_size (sarathi/model_executor/layers/fused_moe/fused_moe.py:346-373

@@ -139,3 +139,31 @@ def fused_moe(hidden_states, w1, w2, gating_output, topk, renormalize):
         down = (act.float() @ w2[e].float().t()) * tw[tok, j].unsqueeze(1)
         parts[tok, j] = down.to(dt)
     return parts.sum(dim=1)
+
+
+def grouped_topk(gating_output, topk, renormalize, num_expert_group, topk_group):
+    """Group-limited routing as the reference states it with tensor ops
+    (sarathi/model_executor/layers/fused_moe/fused_moe.py:377-408): softmax; a group's score is
+    its best member; the topk_group best groups stay, all other experts' scores become 0; top-k.
+    The reference's torch.topk(sorted=False) leaves output order and ties open; this restatement
+    (and the kernel) return descending scores with the lower index first among equals, which is
+    one of the outcomes the reference allows.  Returns (weights f32 [T, k], ids i32 [T, k])."""
+    scores = torch.softmax(gating_output.float(), dim=-1)
+    T, E = scores.shape
+    per_group = E // num_expert_group
+    weights = torch.empty((T, topk), dtype=torch.float32)
+    ids = torch.empty((T, topk), dtype=torch.int32)
+    for t in range(T):
+        row = scores[t]
+        best_of_group = [float(row[g * per_group:(g + 1) * per_group].max())
+                         for g in range(num_expert_group)]
+        order = sorted(range(num_expert_group), key=lambda g: (-best_of_group[g], g))
+        kept = set(order[:topk_group])
+        masked = [float(row[e]) if (e // per_group) in kept else 0.0 for e in range(E)]
+        pick = sorted(range(E), key=lambda e: (-masked[e], e))[:topk]
+        for j, e in enumerate(pick):
+            weights[t, j] = row[e] if (e // per_group) in kept else 0.0
+            ids[t, j] = e
+    if renormalize:
+        weights = weights / weights.sum(dim=-1, keepdim=True)
+    return weights, ids

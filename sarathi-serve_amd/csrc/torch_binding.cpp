@@ -489,6 +489,31 @@ void moe_align_block_size_filled(torch::Tensor topk_ids, int64_t num_experts, in
                  num_tokens_post_pad, true, "moe_align_block_size_filled");
 }
 
+void grouped_topk(torch::Tensor& topk_weights, torch::Tensor& topk_indices,
+                  torch::Tensor& gating_output, int64_t num_expert_group, int64_t topk_group,
+                  bool renormalize) {
+  const char* op = "grouped_topk";
+  check_gpu(gating_output, gating_output, op, "gating_output");
+  check_gpu(topk_weights, gating_output, op, "topk_weights");
+  check_gpu(topk_indices, gating_output, op, "topk_indices");
+  TORCH_CHECK(gating_output.scalar_type() == at::ScalarType::Float &&
+                  topk_weights.scalar_type() == at::ScalarType::Float &&
+                  topk_indices.scalar_type() == at::ScalarType::Int,
+              op, ": gating_output / topk_weights must be float32, topk_indices int32");
+  TORCH_CHECK(gating_output.dim() == 2 && gating_output.is_contiguous() &&
+                  topk_weights.dim() == 2 && topk_weights.is_contiguous() &&
+                  topk_indices.is_contiguous() && topk_weights.size(0) == gating_output.size(0) &&
+                  topk_indices.numel() == topk_weights.numel(),
+              op, ": expected gating_output [T, E], outputs [T, topk], all contiguous");
+  LaunchScope scope(gating_output);
+  raise_on(sarathi_grouped_topk(topk_weights.data_ptr<float>(), topk_indices.data_ptr<int32_t>(),
+                                gating_output.data_ptr<float>(), gating_output.size(0),
+                                (int)gating_output.size(1), (int)topk_weights.size(1),
+                                (int)num_expert_group, (int)topk_group, renormalize ? 1 : 0,
+                                scope.stream),
+           op);
+}
+
 // One zeroed uint32 per (device, stream): the completion counter of the fused routing kernel.
 // Allocated on first use and kept for the life of the process.
 uint32_t* routing_counter(int dev, void* stream) {
@@ -652,6 +677,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "stable sort of token ids by expert, runs padded to block_size");
   m.def("moe_align_block_size_filled", &moe_align_block_size_filled,
         "moe_align_block_size that also writes the padding value into unused slots");
+  m.def("grouped_topk", &grouped_topk,
+        "softmax, keep the best topk_group of num_expert_group expert groups, top-k of the rest");
   m.def("fused_topk_align", &fused_topk_align,
         "topk_softmax (+ optional renormalisation) and moe_align_block_size in one launch");
   m.def("moe_grouped_gemm", &moe_grouped_gemm,

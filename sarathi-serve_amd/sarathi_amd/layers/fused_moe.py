@@ -7,12 +7,15 @@ The two GEMMs are one hand-written MFMA kernel (csrc/moe_gemm.hip) instead of th
 Triton kernel; there are no tuning JSON files, the slot-block size is picked from the batch size.
 fp8 weights / scales are not supported.
 """
-from typing import Any, Dict, Optional
+import functools
+import json
+import os
+from typing import Any, Dict, Optional, Tuple
 
 import torch
 
 from .. import activation_ops, moe_ops
-from .moe_routing import fused_topk, fused_topk_and_align, moe_align_block_size
+from .moe_routing import fused_topk, fused_topk_and_align, grouped_topk, moe_align_block_size
 
 _BLOCK_SIZES = (32, 64, 128, 256)
 
@@ -61,8 +64,53 @@ def get_default_config(M: int, E: int, N: int, K: int, topk: int,
     taller tile re-uses each weight fragment for more tokens).  BLOCK_SIZE_N / BLOCK_SIZE_K are
     fixed properties of the kernel and reported for information."""
     per_expert = M * topk / max(E, 1)
-    block_m = 128 if per_expert >= 384 else 64 if per_expert >= 96 else 32   # 256 measured no faster
+    # thresholds from a sweep of the Mixtral-8x7B shape on MI355X (tune_fused_moe.py); 256 was
+    # never the fastest
+    block_m = 128 if per_expert >= 48 else 64 if per_expert >= 10 else 32
     return {"BLOCK_SIZE_M": block_m, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 64, "GROUP_SIZE_M": 1}
+
+
+def get_config_file_name(E: int, N: int, dtype: Optional[str]) -> str:
+    """Same naming rule as the reference (fused_moe.py:262-265)."""
+    device_name = torch.cuda.get_device_name().replace(" ", "_")
+    dtype_selector = "" if not dtype else f",dtype={dtype}"
+    return f"E={E},N={N},device_name={device_name}{dtype_selector}.json"
+
+
+CONFIG_DIR = os.path.join(os.path.dirname(os.path.realpath(__file__)), "configs")
+
+
+@functools.lru_cache
+def get_moe_configs(E: int, N: int, dtype: Optional[str]) -> Optional[Dict[int, Any]]:
+    """Tuned slot-block sizes for this (E, N) on this device, as a map batch size -> config, or
+    None (reference: fused_moe.py:268-294).  Files are written by ``tune_fused_moe.py``.  MI355X
+    boards report different marketing names depending on the driver, so a file named for the
+    architecture (``device_name=gfx950``) is tried after the one named for the device."""
+    names = [get_config_file_name(E, N, dtype)]
+    arch = getattr(torch.cuda.get_device_properties(torch.cuda.current_device()), "gcnArchName", "")
+    if arch:
+        dtype_selector = "" if not dtype else f",dtype={dtype}"
+        names.append(f"E={E},N={N},device_name={arch.split(':')[0]}{dtype_selector}.json")
+    for name in names:
+        path = os.path.join(CONFIG_DIR, name)
+        if os.path.exists(path):
+            with open(path) as f:
+                return {int(key): val for key, val in json.load(f).items()}
+    return None
+
+
+def try_get_optimal_moe_config(w1_shape: Tuple[int, ...], w2_shape: Tuple[int, ...], top_k: int,
+                               M: int, dtype: Optional[str] = None,
+                               override_config: Optional[Dict[str, Any]] = None) -> Dict[str, Any]:
+    """override_config, else the tuned entry closest to M, else the default rule
+    (reference: fused_moe.py:321-343)."""
+    if override_config:
+        return override_config
+    E, _, N = w2_shape
+    configs = get_moe_configs(E, N, dtype)
+    if configs:
+        return configs[min(configs.keys(), key=lambda x: abs(x - M))]
+    return get_default_config(M, E, N, w1_shape[2], top_k, dtype)
 
 
 def invoke_fused_moe_kernel(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor,
@@ -119,7 +167,8 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
         n = end - begin
         cur_hidden = hidden_states[begin:end]
         cur_ids, cur_w = topk_ids[begin:end], topk_weights[begin:end]
-        config = override_config or get_default_config(n, E, w2.shape[1], K, topk)
+        config = try_get_optimal_moe_config(tuple(w1.shape), tuple(w2.shape), topk, n,
+                                            override_config=override_config)
         c1, c2, c3 = cache1[:n], cache2[:n * topk], cache3[:n]
         if _alignment is not None and n == num_tokens and _alignment[3] == config["BLOCK_SIZE_M"]:
             sorted_ids, expert_ids, post_padded = _alignment[:3]
@@ -145,14 +194,16 @@ def fused_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
     """MoE layer forward: ``hidden_states [T, H]``, ``w1 [E, 2I, H]``, ``w2 [E, H, I]``,
     ``gating_output [T, E]`` (logits)."""
     assert gating_output.shape[1] == w1.shape[0], "Number of experts mismatch"
-    if use_grouped_topk:
-        raise NotImplementedError("grouped_topk (DeepSeek-V2 routing) is not part of this library")
     num_tokens, E = gating_output.shape
     alignment = None
-    if 0 < num_tokens * topk <= FUSED_ROUTING_MAX_SLOTS:
+    if use_grouped_topk:
+        assert num_expert_group is not None and topk_group is not None
+        topk_weights, topk_ids = grouped_topk(hidden_states, gating_output, topk, renormalize,
+                                              num_expert_group, topk_group)
+    elif 0 < num_tokens * topk <= FUSED_ROUTING_MAX_SLOTS:
         # small batches are launch-latency bound: routing and slot sort in one launch
-        config = override_config or get_default_config(num_tokens, E, w2.shape[1],
-                                                       hidden_states.shape[1], topk)
+        config = try_get_optimal_moe_config(tuple(w1.shape), tuple(w2.shape), topk, num_tokens,
+                                            override_config=override_config)
         block_m = config["BLOCK_SIZE_M"]
         topk_weights, topk_ids, sorted_ids, expert_ids, post_padded = fused_topk_and_align(
             hidden_states, gating_output, topk, renormalize, block_m)

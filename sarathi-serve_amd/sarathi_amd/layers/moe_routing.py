@@ -23,6 +23,23 @@ def fused_topk(hidden_states: torch.Tensor, gating_output: torch.Tensor, topk: i
     return topk_weights, topk_ids
 
 
+def grouped_topk(hidden_states: torch.Tensor, gating_output: torch.Tensor, topk: int,
+                 renormalize: bool, num_expert_group: int = 0,
+                 topk_group: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Group-limited routing (DeepSeek-V2): only experts of the ``topk_group`` best of
+    ``num_expert_group`` expert groups can be selected.  Returns (topk_weights f32, topk_ids i32),
+    in descending weight order (the reference's torch.topk(sorted=False) leaves the order open)."""
+    assert hidden_states.shape[0] == gating_output.shape[0], "Number of tokens mismatch"
+    M = hidden_states.shape[0]
+    dev = hidden_states.device
+    topk_weights = torch.empty((M, topk), dtype=torch.float32, device=dev)
+    topk_ids = torch.empty((M, topk), dtype=torch.int32, device=dev)
+    logits = gating_output if gating_output.dtype == torch.float32 else gating_output.float()
+    moe_ops.grouped_topk(topk_weights, topk_ids, logits.contiguous(), num_expert_group, topk_group,
+                         renormalize)
+    return topk_weights, topk_ids
+
+
 def moe_align_block_size(topk_ids: torch.Tensor, block_size: int,
                          num_experts: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Sorts the flat (token, k) slots by expert and pads every expert's run to a multiple of

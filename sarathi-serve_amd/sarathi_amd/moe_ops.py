@@ -18,6 +18,9 @@ moe_grouped_gemm = _C.moe_grouped_gemm
 #                  block_size, sorted_token_ids, experts_ids, num_tokens_post_pad, fill_pad):
 # topk_softmax(_renorm) and moe_align_block_size(_filled) in one launch, same outputs
 fused_topk_align = _C.fused_topk_align
+# grouped_topk(topk_weights, topk_ids, gating_output, num_expert_group, topk_group, renormalize):
+# the group-limited routing the reference writes with tensor ops (fused_moe.py:377-408)
+grouped_topk = _C.grouped_topk
 
 __all__ = ["topk_softmax", "moe_align_block_size", "topk_softmax_renorm",
-           "moe_align_block_size_filled", "moe_grouped_gemm", "fused_topk_align"]
+           "moe_align_block_size_filled", "moe_grouped_gemm", "fused_topk_align", "grouped_topk"]

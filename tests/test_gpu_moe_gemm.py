@@ -126,7 +126,8 @@ def test_fused_moe_forward(ops, dev, T, E, k, H, I, renorm):
 def test_fused_moe_with_one_launch_routing(ops, dev, monkeypatch):
     """fused_moe with the routing + slot sort done by the single fused launch: same bits."""
     from sarathi_amd import layers
-    from sarathi_amd.layers import fused_moe as fm
+    import importlib
+    fm = importlib.import_module("sarathi_amd.layers.fused_moe")   # the module, not the function
     T, E, k, H, I = 300, 8, 2, 256, 512
     g = gen(21)
     x = randn((T, H), g, std=1.0).to(dev)

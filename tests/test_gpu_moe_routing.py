@@ -294,3 +294,24 @@ def test_fused_topk_align_against_oracle(ops, dev):
     assert torch.equal(s.cpu(), os_)
     nb = int(op.item()) // B
     assert torch.equal(e.cpu()[:nb], oe[:nb])
+
+
+# ---- grouped_topk -----------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("T,E,k,G,keep,renorm", [
+    (257, 160, 6, 8, 3, True),       # DeepSeek-V2
+    (64, 16, 4, 1, 1, False),        # one group: plain top-k
+    (100, 64, 8, 64, 8, False),      # groups of one expert
+    (33, 256, 8, 8, 4, True),
+    (50, 1024, 4, 32, 2, False),
+    (7, 6, 3, 3, 2, True),
+])
+def test_grouped_topk_matches_formulation(ops, dev, T, E, k, G, keep, renorm):
+    from oracle import torch_formulations
+    from sarathi_amd import layers
+    gating = torch.randn((T, E), generator=gen(E + k), dtype=torch.float32)
+    ww, wi = torch_formulations.grouped_topk(gating, k, renorm, G, keep)
+    gw, gi = layers.grouped_topk(torch.empty((T, 4), device=dev), gating.to(dev), k, renorm, G, keep)
+    assert gi.dtype == torch.int32 and gw.dtype == torch.float32
+    assert torch.equal(gi.cpu(), wi)
+    assert torch.allclose(gw.cpu(), ww, rtol=0, atol=1e-6)

@@ -636,3 +636,54 @@ def test_paged_kv_round_trip_and_untouched_entries(page_size, before, new):
             written[pages[j // page_size], :, j % page_size] = True
     assert np.array_equal(cache[~written], c["cache"][~written])
     assert not np.array_equal(cache[written], c["cache"][written]) or not written.any()
+
+
+# ---- grouped_topk (oracle/torch_formulations.py) -------------------------------------------------
+
+def test_grouped_topk_single_group_reduces_to_topk_softmax():
+    """One group that is always kept: the routing is plain softmax + top-k, which is pinned above."""
+    from oracle import c_oracle, torch_formulations
+    g = torch.Generator().manual_seed(4)
+    gating = torch.randn((64, 16), generator=g)
+    w, ids = torch_formulations.grouped_topk(gating, 4, False, 1, 1)
+    ww = torch.empty((64, 4)); wi = torch.empty((64, 4), dtype=torch.int32)
+    ws = torch.empty((64, 4), dtype=torch.int32)
+    c_oracle.topk_softmax(ww, wi, ws, gating)
+    assert torch.equal(ids, wi) and torch.allclose(w, ww, rtol=0, atol=1e-6)
+
+
+def test_grouped_topk_hand_worked_example():
+    """6 experts in 3 groups of 2, keep 2 groups, top-3.  Logits chosen so that the probabilities
+    order as e4 > e1 > e5 > e0 > e2 > e3: groups score (e1, e2, e4) -> groups 2 and 0 stay, group 1
+    (e2, e3) is masked, and the three best of {e0, e1, e4, e5} are e4, e1, e5."""
+    from oracle import torch_formulations
+    logits = torch.tensor([[1.0, 3.0, 0.5, 0.0, 4.0, 2.0]])
+    w, ids = torch_formulations.grouped_topk(logits, 3, False, 3, 2)
+    assert ids.tolist() == [[4, 1, 5]]
+    p = torch.softmax(logits, dim=-1)[0]
+    assert torch.allclose(w[0], p[[4, 1, 5]])
+    # keeping a single group: e4's group (e4, e5) only; the third pick is a masked expert with
+    # weight 0, the lowest index among them
+    w1, ids1 = torch_formulations.grouped_topk(logits, 3, False, 3, 1)
+    assert ids1.tolist() == [[4, 5, 0]] and w1[0, 2].item() == 0.0
+    # renormalised weights sum to one
+    wr, _ = torch_formulations.grouped_topk(logits, 3, True, 3, 2)
+    assert abs(float(wr.sum()) - 1.0) < 1e-6
+
+
+def test_grouped_topk_selected_experts_stay_inside_the_kept_groups():
+    from oracle import torch_formulations
+    g = torch.Generator().manual_seed(9)
+    gating = torch.randn((200, 160), generator=g)
+    w, ids = torch_formulations.grouped_topk(gating, 6, True, 8, 3)      # DeepSeek-V2 shape
+    p = torch.softmax(gating, dim=-1)
+    for t in range(200):
+        groups = set((ids[t] // 20).tolist())
+        assert len(groups) <= 3
+        gs = p[t].view(8, 20).max(dim=-1).values
+        kept = set(torch.topk(gs, 3).indices.tolist())
+        assert groups <= kept
+        # nothing better was left behind inside the kept groups
+        inside = torch.tensor([e for e in range(160) if e // 20 in kept])
+        assert torch.equal(torch.sort(ids[t].long()).values,
+                           torch.sort(inside[torch.topk(p[t][inside], 6).indices]).values)
