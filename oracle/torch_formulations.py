@@ -115,18 +115,22 @@ def moe_grouped_gemm(A, B, C, topk_weights, sorted_token_ids, expert_ids, num_to
         Cf[slots] = acc.to(C.dtype)
 
 
-def fused_moe(hidden_states, w1, w2, gating_output, topk, renormalize):
+def fused_moe(hidden_states, w1, w2, gating_output, topk, renormalize, topk_weights=None,
+              topk_ids=None):
     """Dense statement of the MoE layer the reference's fused_moe computes (fused_moe.py:411-622),
     keeping its intermediate tensors in the model dtype: out[t] = sum_j T(w_j * (h_j @ W2[e_j]^T))
     with h_j = silu_and_mul(T(x_t @ W1[e_j]^T))."""
     T, _ = hidden_states.shape
     dt = hidden_states.dtype
-    tw = torch.empty((T, topk), dtype=torch.float32)
-    ti = torch.empty((T, topk), dtype=torch.int32)
-    ts = torch.empty((T, topk), dtype=torch.int32)
-    topk_softmax(tw, ti, ts, gating_output.float())
-    if renormalize:
-        tw = tw / tw.sum(dim=-1, keepdim=True)
+    if topk_ids is not None:      # routing decided by the caller (e.g. grouped_topk)
+        tw, ti = topk_weights, topk_ids
+    else:
+        tw = torch.empty((T, topk), dtype=torch.float32)
+        ti = torch.empty((T, topk), dtype=torch.int32)
+        ts = torch.empty((T, topk), dtype=torch.int32)
+        topk_softmax(tw, ti, ts, gating_output.float())
+        if renormalize:
+            tw = tw / tw.sum(dim=-1, keepdim=True)
     inter = w1.shape[1] // 2
     parts = torch.zeros((T, topk, w2.shape[1]), dtype=dt)
     for e in range(w1.shape[0]):

@@ -138,3 +138,51 @@ def test_fused_moe_with_one_launch_routing(ops, dev, monkeypatch):
     monkeypatch.setattr(fm, "FUSED_ROUTING_MAX_SLOTS", 16384)
     got = layers.fused_moe(x, w1, w2, gating, k, True)
     assert torch.equal(got, want)
+
+
+def test_tuned_config_lookup_and_override(ops, dev):
+    """The Mixtral-8x7B table shipped with the package is found on this device and the entry
+    nearest to the batch size is used; override_config wins; unknown shapes use the default rule."""
+    from sarathi_amd import layers
+    table = layers.get_moe_configs(8, 14336, None)
+    assert table is not None and 4096 in table and table[4096]["BLOCK_SIZE_M"] in (32, 64, 128, 256)
+    w1_shape, w2_shape = (8, 28672, 4096), (8, 4096, 14336)
+    assert layers.try_get_optimal_moe_config(w1_shape, w2_shape, 2, 3000) == table[3072]
+    assert layers.try_get_optimal_moe_config(w1_shape, w2_shape, 2, 5) == table[4]
+    forced = {"BLOCK_SIZE_M": 32}
+    assert layers.try_get_optimal_moe_config(w1_shape, w2_shape, 2, 3000,
+                                             override_config=forced) is forced
+    assert layers.get_moe_configs(7, 1234, None) is None
+    assert layers.try_get_optimal_moe_config((7, 2468, 64), (7, 64, 1234), 2, 512) == \
+        layers.get_default_config(512, 7, 1234, 64, 2)
+
+
+@pytest.mark.parametrize("grouped", [False, True])
+def test_fused_moe_module(ops, dev, grouped):
+    """The FusedMoE module (weights as parameters, in-place forward) against the dense CPU
+    formulation, with row-major and with packed weights."""
+    from sarathi_amd import layers
+    T, E, k, H, I = 200, 8, 2, 256, 512
+    g = gen(31)
+    layer = layers.FusedMoE(E, k, H, I, params_dtype=torch.bfloat16, renormalize=True,
+                            use_grouped_topk=grouped, num_expert_group=4 if grouped else None,
+                            topk_group=2 if grouped else None)
+    assert layer.w13_weight.shape == (E, 2 * I, H) and layer.w2_weight.shape == (E, H, I)
+    w1 = randn((E, 2 * I, H), g, std=H ** -0.5)
+    w2 = randn((E, H, I), g, std=I ** -0.5)
+    layer.w13_weight.data.copy_(w1)
+    layer.w2_weight.data.copy_(w2)
+    x = randn((T, H), g, std=1.0)
+    logits = torch.randn((T, E), generator=g, dtype=torch.float32)
+    if grouped:
+        tw, ti = torch_formulations.grouped_topk(logits, k, True, 4, 2)
+        want = torch_formulations.fused_moe(x, w1, w2, logits, k, True, topk_weights=tw, topk_ids=ti)
+    else:
+        want = torch_formulations.fused_moe(x, w1, w2, logits, k, True)
+    xd = x.to(dev)
+    out = layer(xd, logits.to(dev))
+    assert out.data_ptr() == xd.data_ptr()
+    _close(out, want, "FusedMoE")
+    layer.pack_weights()
+    out2 = layer(x.to(dev), logits.to(dev))
+    assert torch.equal(out2, out)
