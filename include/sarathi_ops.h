@@ -200,8 +200,14 @@ int sarathi_fused_topk_align(float* topk_weights, int32_t* topk_indices,
  * (sarathi/model_executor/layers/fused_moe/fused_moe.py:15-148, :207-260).
  * For every block of block_m consecutive slots of sorted_token_ids (one expert,
  * expert_ids[block]):  C[slot, :] = A[slot / top_k, :] @ B[expert]^T, fp32
- * accumulation, times topk_weights[slot] when mul_routed_weight != 0, rounded
- * to `dtype`.  A [tokens, K] with rows a_row_stride elements apart, B
+ * accumulation, then the epilogue, rounded to `dtype`.  Epilogues:
+ *   SARATHI_MOE_EPILOGUE_NONE           nothing (the reference's mul_routed_weight = False)
+ *   SARATHI_MOE_EPILOGUE_ROUTED_WEIGHT  times topk_weights[slot] (mul_routed_weight = True)
+ *   SARATHI_MOE_EPILOGUE_SILU_AND_MUL   (new) B holds gate rows [0, N/2) and up rows [N/2, N); C is
+ *       [num_valid_tokens, N/2] = silu_and_mul of the [.., N] product, with the rounding points
+ *       of the unfused sequence GEMM -> silu_and_mul (fused_moe.py:499-520), so results are
+ *       bit-identical to it while the [.., N] intermediate never reaches memory.  N/2 must be a
+ *       multiple of 4 (of 32 with packed weights).  A [tokens, K] with rows a_row_stride elements apart, B
  * [E, N, K] K-contiguous with experts b_expert_stride elements apart, C
  * [num_valid_tokens, N] with rows c_row_stride apart (num_valid_tokens =
  * tokens * topk; slots holding a larger id are padding and skipped).
@@ -217,13 +223,15 @@ int sarathi_fused_topk_align(float* topk_weights, int32_t* topk_indices,
  */
 #define SARATHI_MOE_B_ROW_MAJOR 0
 #define SARATHI_MOE_B_PACKED 1
+#define SARATHI_MOE_EPILOGUE_NONE 0
+#define SARATHI_MOE_EPILOGUE_ROUTED_WEIGHT 1
+#define SARATHI_MOE_EPILOGUE_SILU_AND_MUL 2
 int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c, const float* topk_weights,
                              const int32_t* sorted_token_ids, const int32_t* expert_ids,
                              const int32_t* num_tokens_post_padded, int64_t num_valid_tokens,
                              int64_t sorted_len, int64_t n, int64_t k, int64_t a_row_stride,
                              int64_t b_expert_stride, int64_t c_row_stride, int block_m,
-                             int top_k, int mul_routed_weight, int b_layout, int dtype,
-                             void* stream);
+                             int top_k, int epilogue, int b_layout, int dtype, void* stream);
 
 /*
  * Paged KV cache (NHD page layout: entry e of page p holds [num_kv_heads, head_size] elements and

@@ -40,7 +40,7 @@ def main():
     w1 = (torch.randn((E, 2 * I, H), device=dev, dtype=torch.float32) * H ** -0.5).to(bf)
     w2 = (torch.randn((E, H, I), device=dev, dtype=torch.float32) * I ** -0.5).to(bf)
     gating = torch.randn((T, E), device=dev, dtype=torch.float32)
-    config = get_default_config(T, E, H, H, k)
+    config = dict(get_default_config(T, E, I, H, k))
     if args.block_m:
         config["BLOCK_SIZE_M"] = args.block_m
     bm = config["BLOCK_SIZE_M"]
@@ -77,13 +77,20 @@ def main():
             b1, b2, pk, wa, wb = w1, w2, False, w1, w2
         g1 = lambda: ops.moe_ops.moe_grouped_gemm(x, b1, c1, tw, s, e, p, T * k, bm, k, False, pk, 2 * I)  # noqa: E731
         g2 = lambda: ops.moe_ops.moe_grouped_gemm(c2, b2, c3, tw, s, e, p, T * k, bm, 1, True, pk, H)  # noqa: E731
+        g1s = lambda: ops.moe_ops.moe_grouped_gemm(x, b1, c2, tw, s, e, p, T * k, bm, k, False, pk, 2 * I, True)  # noqa: E731
         ms1 = timeit(g1)
+        ms_act = timeit(lambda: ops.activation_ops.silu_and_mul(c2, c1.view(-1, 2 * I)))
+        ms1s = timeit(g1s)
         ops.activation_ops.silu_and_mul(c2, c1.view(-1, 2 * I))
         ms2 = timeit(g2)
         ms_all = timeit(lambda: layers.fused_moe(x, wa, wb, gating, k, True, override_config=config))
         res[label] = {
             "gemm_w1": {"ms": round(ms1, 4), "TFLOPs": round(f1 / ms1 * 1e-9, 1),
                         "frac_of_mfma_peak": round(f1 / ms1 * 1e-9 / MFMA_PEAK_TFLOPS, 4)},
+            "silu_and_mul": {"ms": round(ms_act, 4)},
+            "gemm_w1_with_silu_and_mul_epilogue": {
+                "ms": round(ms1s, 4), "TFLOPs": round(f1 / ms1s * 1e-9, 1),
+                "frac_of_mfma_peak": round(f1 / ms1s * 1e-9 / MFMA_PEAK_TFLOPS, 4)},
             "gemm_w2": {"ms": round(ms2, 4), "TFLOPs": round(f2 / ms2 * 1e-9, 1),
                         "frac_of_mfma_peak": round(f2 / ms2 * 1e-9 / MFMA_PEAK_TFLOPS, 4)},
             "fused_moe_forward": {"ms": round(ms_all, 4),

@@ -25,12 +25,6 @@ namespace sarathi_hip {
 constexpr int kActBlock = 256;   // element-wise fallback kernels
 constexpr int kRowSeg = 64;      // lanes per workgroup of the streaming kernels
 
-SK_DEV float silu_f32(float x) {
-  // x * sigmoid(x) = x / (1 + 2^(-x * log2 e))
-  float e = __builtin_amdgcn_exp2f(x * -1.4426950408889634f);
-  return x * __builtin_amdgcn_rcpf(1.0f + e);
-}
-
 // tanh(u) = 1 - 2 / (1 + e^{2u}); the clamp keeps e^{2u} finite
 SK_DEV float tanh_f32(float u) {
   float c = u < -15.f ? -15.f : (u > 15.f ? 15.f : u);  // NaN passes through

@@ -31,6 +31,12 @@
 //            (BM x 64 elements, 16-byte chunks rotated by row so that the
 //            operand reads are bank-conflict free), double buffered, one
 //            barrier per K-step.
+// Epilogues: plain; times the slot's routing weight (the down projection); or gated SiLU (the
+// gate/up projection followed by silu_and_mul, fused_moe.py:499-520): B then holds the gate rows
+// [0, N/2) and the up rows [N/2, N), a wave takes 32 gate rows and the 32 matching up rows as
+// its two weight tiles, so gate and up of an output element sit in the same lane, and
+// C [slots, N/2] = T(T(silu(T(gate))) * T(up)) is written directly: bit-identical to the
+// unfused pair of kernels, without the [slots, N] intermediate ever reaching memory.
 // Workgroup ids are mapped so that the eight XCDs (id mod 8) each take their
 // own column blocks and walk the slot blocks fastest: workgroups that run
 // together on an XCD share the expert's weight tile in that XCD's L2.
@@ -46,6 +52,8 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 constexpr int kGemmBN = 256;   // output columns per workgroup
 constexpr int kGemmBK = 64;    // K elements per pipeline step
 constexpr int kGemmWaveN = 64; // output columns per wave
+
+enum : int { kEpiPlain = 0, kEpiMulWeight = 1, kEpiGatedSilu = 2 };
 
 template <int DT> SK_DEV f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
   if constexpr (DT == kBF16)
@@ -85,8 +93,15 @@ struct MoeGemmArgs {
 // BM slots per workgroup = WM wave rows x (BM / WM) slots; four wave columns of 64 output columns.
 // WM = 2 (BM = 256, eight waves) halves the number of times a weight tile is pulled out of L2,
 // which is what bounds this kernel once the loads are coalesced.
-template <int DT, int BM, int WM, bool MUL_WEIGHT, bool PACKED>
-__global__ __launch_bounds__(256 * WM) void moe_gemm_kernel(MoeGemmArgs g) {
+// At least two waves per SIMD: with 128 accumulator registers per lane (BM = 128 / 256) that
+// caps the other registers at 128, which the main loop meets anyway (106); without the bound
+// the epilogues that do arithmetic on the accumulators are allocated ~138 and the whole kernel
+// drops to one wave per SIMD (measured: 15 % slower).
+template <int DT, int BM, int WM, int EPI, bool PACKED>
+__global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(2)))
+void moe_gemm_kernel(MoeGemmArgs g) {
+  constexpr bool MUL_WEIGHT = EPI == kEpiMulWeight;
+  constexpr bool GATED = EPI == kEpiGatedSilu;
   constexpr int THREADS = 256 * WM;
   constexpr int MT = BM / WM / 32;     // token tiles per wave
   constexpr int NT = kGemmWaveN / 32;  // weight tiles per wave
@@ -110,7 +125,10 @@ __global__ __launch_bounds__(256 * WM) void moe_gemm_kernel(MoeGemmArgs g) {
   const int l32 = lane & 31, grp = lane >> 5;
 
   // ---- weights: buffer resource over the expert's matrix; rows >= N read as zero
-  const int n_wave0 = pid_n * kGemmBN + wave * kGemmWaveN;
+  // first weight row (= output column) of this wave; gated: first GATE row, 32 per wave
+  const int n_wave0 = GATED ? pid_n * (kGemmBN / 2) + wave * (kGemmWaveN / 2)
+                            : pid_n * kGemmBN + wave * kGemmWaveN;
+  const int half_n = g.N >> 1;  // gated: rows [half_n, N) are the up projection
   const int n_tiles = (g.N + 31) >> 5;
   const int64_t b_bytes = PACKED ? (int64_t)n_tiles * 32 * g.K * 2 : (int64_t)g.N * g.K * 2;
   const rsrc_t rb = make_rsrc(reinterpret_cast<const char*>(g.b) + (int64_t)expert * g.b_expert_stride * 2,
@@ -118,12 +136,17 @@ __global__ __launch_bounds__(256 * WM) void moe_gemm_kernel(MoeGemmArgs g) {
   uint32_t w_off[NT];  // byte offset of this lane's operand piece at k = 0
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
+    // first weight row of tile nt; gated: tile 0 = gate rows, tile 1 = the matching up rows
+    const int n_tile0 = GATED ? n_wave0 + nt * half_n : n_wave0 + nt * 32;
+    const bool live = GATED ? n_wave0 < half_n : true;
     if constexpr (PACKED) {
-      const int tile = (n_wave0 >> 5) + nt;  // 32-row tile; its K/16 operand blocks of 1 KiB follow each other
-      w_off[nt] = tile < n_tiles ? (uint32_t)tile * (uint32_t)g.K * 64u + lane * 16u : 0x80000000u;
+      const int tile = n_tile0 >> 5;  // 32-row tile; its K/16 operand blocks of 1 KiB follow each other
+      w_off[nt] = live && tile < n_tiles ? (uint32_t)tile * (uint32_t)g.K * 64u + lane * 16u
+                                         : 0x80000000u;
     } else {
-      const int n = n_wave0 + nt * 32 + l32;
-      w_off[nt] = n < g.N ? (uint32_t)n * (uint32_t)g.K * 2u + grp * 16u : 0x80000000u;
+      const int n = n_tile0 + l32;
+      const bool in_range = GATED ? n_wave0 + l32 < half_n : n < g.N;
+      w_off[nt] = live && in_range ? (uint32_t)n * (uint32_t)g.K * 2u + grp * 16u : 0x80000000u;
     }
   }
   // operand piece of sub-step s (16 deep) of the K-step starting at k0
@@ -228,22 +251,43 @@ __global__ __launch_bounds__(256 * WM) void moe_gemm_kernel(MoeGemmArgs g) {
     float scale = 1.f;
     if constexpr (MUL_WEIGHT) scale = g.topk_weights[sid];
     char* crow = reinterpret_cast<char*>(g.c) + (int64_t)sid * g.c_row_stride * 2;
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
+    if constexpr (GATED) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int n = n_wave0 + nt * 32 + q * 8 + grp * 4;
-        float v0 = acc[nt][mt][q * 4 + 0], v1 = acc[nt][mt][q * 4 + 1];
-        float v2 = acc[nt][mt][q * 4 + 2], v3 = acc[nt][mt][q * 4 + 3];
-        if constexpr (MUL_WEIGHT) { v0 *= scale; v1 *= scale; v2 *= scale; v3 *= scale; }
-        if (n + 3 < g.N) {
-          u32x2 out = {pack2<DT>(v0, v1), pack2<DT>(v2, v3)};
+        const int n = n_wave0 + q * 8 + grp * 4;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float x = rnd<DT>(acc[0][mt][q * 4 + e]), y = rnd<DT>(acc[1][mt][q * 4 + e]);
+          v[e] = rnd<DT>(silu_f32(x)) * y;
+        }
+        if (n + 3 < half_n) {
+          u32x2 out = {pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
           *reinterpret_cast<u32x2*>(crow + (int64_t)n * 2) = out;
         } else {
-          const float v[4] = {v0, v1, v2, v3};
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            if (n + e < g.N) store_elem<DT>(crow, n + e, v[e]);
+            if (n + e < half_n) store_elem<DT>(crow, n + e, v[e]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = n_wave0 + nt * 32 + q * 8 + grp * 4;
+          float v0 = acc[nt][mt][q * 4 + 0], v1 = acc[nt][mt][q * 4 + 1];
+          float v2 = acc[nt][mt][q * 4 + 2], v3 = acc[nt][mt][q * 4 + 3];
+          if constexpr (MUL_WEIGHT) { v0 *= scale; v1 *= scale; v2 *= scale; v3 *= scale; }
+          if (n + 3 < g.N) {
+            u32x2 out = {pack2<DT>(v0, v1), pack2<DT>(v2, v3)};
+            *reinterpret_cast<u32x2*>(crow + (int64_t)n * 2) = out;
+          } else {
+            const float v[4] = {v0, v1, v2, v3};
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n + e < g.N) store_elem<DT>(crow, n + e, v[e]);
+          }
         }
       }
     }
@@ -251,16 +295,21 @@ __global__ __launch_bounds__(256 * WM) void moe_gemm_kernel(MoeGemmArgs g) {
 }
 
 template <int DT, int BM>
-static int launch_moe_gemm(const MoeGemmArgs& g, bool mul_weight, bool packed, hipStream_t st) {
+static int launch_moe_gemm(const MoeGemmArgs& g, int epilogue, bool packed, hipStream_t st) {
   constexpr int WM = BM > 128 ? 2 : 1;
   const int64_t groups = (g.n_blocks + 7) / 8;
   const int64_t blocks = groups * g.m_blocks * 8;
   if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)blocks), block(256 * WM);
-#define SK_LAUNCH(MW, PK) \
-  hipLaunchKernelGGL((moe_gemm_kernel<DT, BM, WM, MW, PK>), grid, block, 0, st, g)
-  if (mul_weight) { if (packed) SK_LAUNCH(true, true); else SK_LAUNCH(true, false); }
-  else { if (packed) SK_LAUNCH(false, true); else SK_LAUNCH(false, false); }
+#define SK_LAUNCH(EP, PK) \
+  hipLaunchKernelGGL((moe_gemm_kernel<DT, BM, WM, EP, PK>), grid, block, 0, st, g)
+  if (epilogue == kEpiMulWeight) {
+    if (packed) SK_LAUNCH(kEpiMulWeight, true); else SK_LAUNCH(kEpiMulWeight, false);
+  } else if (epilogue == kEpiGatedSilu) {
+    if (packed) SK_LAUNCH(kEpiGatedSilu, true); else SK_LAUNCH(kEpiGatedSilu, false);
+  } else {
+    if (packed) SK_LAUNCH(kEpiPlain, true); else SK_LAUNCH(kEpiPlain, false);
+  }
 #undef SK_LAUNCH
   return launch_status();
 }
@@ -275,14 +324,21 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
                                         int64_t num_valid_tokens, int64_t sorted_len, int64_t n,
                                         int64_t k, int64_t a_row_stride, int64_t b_expert_stride,
                                         int64_t c_row_stride, int block_m, int top_k,
-                                        int mul_routed_weight, int b_layout, int dtype,
+                                        int epilogue, int b_layout, int dtype,
                                         void* stream) {
   using namespace sarathi_hip;
   if (!a || !b || !c || !sorted_token_ids || !expert_ids || !num_tokens_post_padded)
     return SARATHI_ERR_INVALID_ARG;
-  if (mul_routed_weight && !topk_weights) return SARATHI_ERR_INVALID_ARG;
+  if (epilogue != SARATHI_MOE_EPILOGUE_NONE && epilogue != SARATHI_MOE_EPILOGUE_ROUTED_WEIGHT &&
+      epilogue != SARATHI_MOE_EPILOGUE_SILU_AND_MUL)
+    return SARATHI_ERR_INVALID_ARG;
+  if (epilogue == SARATHI_MOE_EPILOGUE_ROUTED_WEIGHT && !topk_weights)
+    return SARATHI_ERR_INVALID_ARG;
+  const bool gated = epilogue == SARATHI_MOE_EPILOGUE_SILU_AND_MUL;
+  if (gated && (n & 1)) return SARATHI_ERR_INVALID_ARG;
+  const int64_t c_cols = gated ? n / 2 : n;  // width of C
   if (num_valid_tokens < 0 || sorted_len < 0 || n <= 0 || k <= 0 || top_k <= 0 ||
-      a_row_stride < k || c_row_stride < n || b_expert_stride < n * k ||
+      a_row_stride < k || c_row_stride < c_cols || b_expert_stride < n * k ||
       (b_layout != SARATHI_MOE_B_ROW_MAJOR && b_layout != SARATHI_MOE_B_PACKED))
     return SARATHI_ERR_INVALID_ARG;
   const bool packed = b_layout == SARATHI_MOE_B_PACKED;
@@ -294,6 +350,8 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
   if (k % kGemmBK != 0 || a_row_stride % 8 != 0 || b_expert_stride % 8 != 0 || n % 4 != 0 ||
       c_row_stride % 4 != 0 || !aligned16(a) || !aligned16(b) || (reinterpret_cast<uintptr_t>(c) & 7u))
     return SARATHI_ERR_UNSUPPORTED;
+  // gated: output pieces of 4 columns; packed tiles of 32 rows must not straddle gate and up
+  if (gated && (c_cols % 4 != 0 || (packed && c_cols % 32 != 0))) return SARATHI_ERR_UNSUPPORTED;
   if ((n + 31) / 32 * 32 * k * 2 >= 0x80000000LL || num_valid_tokens > 0x7fffffffLL || sorted_len > 0x7fffffffLL)
     return SARATHI_ERR_UNSUPPORTED;
   // A is addressed through one buffer resource with 32-bit offsets
@@ -316,9 +374,10 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
   g.N = (int32_t)n; g.K = (int32_t)k;
   g.top_k = top_k;
   g.m_blocks = (int32_t)((sorted_len + block_m - 1) / block_m);
-  g.n_blocks = (int32_t)((n + kGemmBN - 1) / kGemmBN);
+  g.n_blocks = gated ? (int32_t)((c_cols + kGemmBN / 2 - 1) / (kGemmBN / 2))
+                     : (int32_t)((n + kGemmBN - 1) / kGemmBN);
   hipStream_t st = (hipStream_t)stream;
-  const bool mw = mul_routed_weight != 0;
+  const int mw = epilogue;
 #define SK_GEMM(DT)                                                       \
   switch (block_m) {                                                      \
     case 32: return launch_moe_gemm<DT, 32>(g, mw, packed, st);           \

@@ -582,7 +582,7 @@ void moe_grouped_gemm(torch::Tensor& a, torch::Tensor& b, torch::Tensor& c,
                       torch::Tensor& topk_weights, torch::Tensor& sorted_token_ids,
                       torch::Tensor& expert_ids, torch::Tensor& num_tokens_post_padded,
                       int64_t num_valid_tokens, int64_t block_m, int64_t top_k,
-                      bool mul_routed_weight, bool b_packed, int64_t n) {
+                      bool mul_routed_weight, bool b_packed, int64_t n, bool silu_and_mul) {
   const char* op = "moe_grouped_gemm";
   check_gpu(a, a, op, "A");
   check_gpu(b, a, op, "B");
@@ -609,8 +609,12 @@ void moe_grouped_gemm(torch::Tensor& a, torch::Tensor& b, torch::Tensor& c,
               ": A, B and C must share a dtype");
   TORCH_CHECK(a.scalar_type() == at::ScalarType::BFloat16 || a.scalar_type() == at::ScalarType::Half,
               op, ": only bfloat16 and float16 are supported");
-  TORCH_CHECK(c.is_contiguous() && c.size(-1) == n && c.numel() == num_valid_tokens * n, op,
-              ": C must be contiguous and hold num_valid_tokens rows of N elements");
+  TORCH_CHECK(!(silu_and_mul && mul_routed_weight), op,
+              ": silu_and_mul and mul_routed_weight are different epilogues; pick one");
+  TORCH_CHECK(!silu_and_mul || n % 2 == 0, op, ": silu_and_mul needs an even N (gate rows, up rows)");
+  const int64_t c_cols = silu_and_mul ? n / 2 : n;
+  TORCH_CHECK(c.is_contiguous() && c.size(-1) == c_cols && c.numel() == num_valid_tokens * c_cols,
+              op, ": C must be contiguous and hold num_valid_tokens rows of ", c_cols, " elements");
   TORCH_CHECK(topk_weights.scalar_type() == at::ScalarType::Float && topk_weights.is_contiguous() &&
                   topk_weights.numel() >= (mul_routed_weight ? num_valid_tokens : 0),
               op, ": topk_weights must be contiguous float32 [tokens, topk]");
@@ -626,8 +630,11 @@ void moe_grouped_gemm(torch::Tensor& a, torch::Tensor& b, torch::Tensor& c,
                a.data_ptr(), b.data_ptr(), c.data_ptr(), topk_weights.data_ptr<float>(),
                sorted_token_ids.data_ptr<int32_t>(), expert_ids.data_ptr<int32_t>(),
                num_tokens_post_padded.data_ptr<int32_t>(), num_valid_tokens,
-               sorted_token_ids.numel(), n, k, a.stride(0), expert_stride, n, (int)block_m,
-               (int)top_k, mul_routed_weight ? 1 : 0,
+               sorted_token_ids.numel(), n, k, a.stride(0), expert_stride, c_cols, (int)block_m,
+               (int)top_k,
+               silu_and_mul ? SARATHI_MOE_EPILOGUE_SILU_AND_MUL
+                            : mul_routed_weight ? SARATHI_MOE_EPILOGUE_ROUTED_WEIGHT
+                                                : SARATHI_MOE_EPILOGUE_NONE,
                b_packed ? SARATHI_MOE_B_PACKED : SARATHI_MOE_B_ROW_MAJOR, dtype_code(a, op),
                scope.stream),
            op);
@@ -687,5 +694,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         pybind11::arg("sorted_token_ids"), pybind11::arg("expert_ids"),
         pybind11::arg("num_tokens_post_padded"), pybind11::arg("num_valid_tokens"),
         pybind11::arg("block_m"), pybind11::arg("top_k"), pybind11::arg("mul_routed_weight"),
-        pybind11::arg("b_packed") = false, pybind11::arg("n") = 0);
+        pybind11::arg("b_packed") = false, pybind11::arg("n") = 0,
+        pybind11::arg("silu_and_mul") = false);
 }

@@ -97,6 +97,14 @@ template <int DT> struct Vec {
   }
 };
 
+// ---- activation shared by silu_and_mul and the gated GEMM epilogue ---------------------------
+
+SK_DEV float silu_f32(float x) {
+  // x * sigmoid(x) = x / (1 + 2^(-x * log2 e))
+  float e = __builtin_amdgcn_exp2f(x * -1.4426950408889634f);
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
 // ---- global memory ---------------------------------------------------------
 
 // 16-byte accesses go through raw buffer instructions: the base pointer of the

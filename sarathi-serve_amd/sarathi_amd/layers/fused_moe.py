@@ -55,6 +55,8 @@ def pack_expert_weights(w: torch.Tensor) -> PackedExpertWeights:
 # ids through device-coherent loads, which costs what the saved launch gains); it only pays when
 # the host, not the GPU, is the bottleneck of the launch sequence.
 FUSED_ROUTING_MAX_SLOTS = 0
+# silu_and_mul inside the gate/up GEMM's epilogue (same bits as the separate kernel)
+FUSE_SILU_AND_MUL = True
 CHUNK_SIZE = 64 * 1024     # tokens per pass, as in the reference (fused_moe.py:437)
 
 
@@ -118,9 +120,12 @@ def invoke_fused_moe_kernel(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor,
                             topk_weights: torch.Tensor, topk_ids: torch.Tensor,
                             sorted_token_ids: torch.Tensor, expert_ids: torch.Tensor,
                             num_tokens_post_padded: torch.Tensor, mul_routed_weight: bool,
-                            top_k: int, config: Dict[str, Any], compute_type=None) -> None:
+                            top_k: int, config: Dict[str, Any], compute_type=None,
+                            silu_and_mul: bool = False) -> None:
     """Same argument list as the reference's launcher.  ``config["BLOCK_SIZE_M"]`` must be the block
-    size ``sorted_token_ids`` was aligned with."""
+    size ``sorted_token_ids`` was aligned with.  ``silu_and_mul=True`` (not in the reference):
+    ``B`` is a gate/up projection ``[E, 2I, K]`` and ``C [.., I]`` receives
+    ``silu_and_mul(A @ B^T)`` directly, bit-identical to running the two ops separately."""
     assert A_scale is None and B_scale is None, "fp8 scales are not supported"
     assert topk_weights.stride(1) == 1 and sorted_token_ids.stride(0) == 1
     block_m = int(config["BLOCK_SIZE_M"])
@@ -129,7 +134,7 @@ def invoke_fused_moe_kernel(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor,
     packed = isinstance(B, PackedExpertWeights)
     moe_ops.moe_grouped_gemm(A, B.data if packed else B, C, topk_weights, sorted_token_ids,
                              expert_ids, num_tokens_post_padded, topk_ids.numel(), block_m, top_k,
-                             bool(mul_routed_weight), packed, B.shape[1])
+                             bool(mul_routed_weight), packed, B.shape[1], bool(silu_and_mul))
 
 
 def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
@@ -157,7 +162,9 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
     while chunk > 1 and max(chunk * K, chunk * topk * (N // 2)) * eb + 4 * max(K, N) >= 1 << 32:
         chunk //= 2
     M = min(num_tokens, chunk)
-    cache1 = torch.empty((M, topk, N), device=dev, dtype=dt)
+    # gate/up GEMM with the activation fused into its epilogue: no [M, topk, N] intermediate
+    fuse_act = FUSE_SILU_AND_MUL and (N // 2) % 32 == 0
+    cache1 = None if fuse_act else torch.empty((M, topk, N), device=dev, dtype=dt)
     cache2 = torch.empty((M * topk, N // 2), device=dev, dtype=dt)
     cache3 = torch.empty((M, topk, w2.shape[1]), device=dev, dtype=dt)
     out = hidden_states if inplace else torch.empty_like(hidden_states)
@@ -169,15 +176,21 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
         cur_ids, cur_w = topk_ids[begin:end], topk_weights[begin:end]
         config = try_get_optimal_moe_config(tuple(w1.shape), tuple(w2.shape), topk, n,
                                             override_config=override_config)
-        c1, c2, c3 = cache1[:n], cache2[:n * topk], cache3[:n]
+        c2, c3 = cache2[:n * topk], cache3[:n]
         if _alignment is not None and n == num_tokens and _alignment[3] == config["BLOCK_SIZE_M"]:
             sorted_ids, expert_ids, post_padded = _alignment[:3]
         else:
             sorted_ids, expert_ids, post_padded = moe_align_block_size(
                 cur_ids, config["BLOCK_SIZE_M"], E)
-        invoke_fused_moe_kernel(cur_hidden, w1, c1, None, None, cur_w, cur_ids, sorted_ids,
-                                expert_ids, post_padded, False, topk, config)
-        activation_ops.silu_and_mul(c2, c1.view(-1, N))
+        if fuse_act:
+            invoke_fused_moe_kernel(cur_hidden, w1, c2, None, None, cur_w, cur_ids, sorted_ids,
+                                    expert_ids, post_padded, False, topk, config,
+                                    silu_and_mul=True)
+        else:
+            c1 = cache1[:n]
+            invoke_fused_moe_kernel(cur_hidden, w1, c1, None, None, cur_w, cur_ids, sorted_ids,
+                                    expert_ids, post_padded, False, topk, config)
+            activation_ops.silu_and_mul(c2, c1.view(-1, N))
         invoke_fused_moe_kernel(c2, w2, c3, None, None, cur_w, cur_ids, sorted_ids, expert_ids,
                                 post_padded, True, 1, config)
         torch.sum(c3, dim=1, out=out[begin:end])

@@ -194,6 +194,8 @@ def test_kv_cache_and_gemm_argument_validation_without_gpu(lib):
     assert gemm(w=null, mul=1) == INVALID           # routing weights required when multiplying
     assert gemm(astride=32) == INVALID              # rows of A narrower than K
     assert gemm(layout=5) == INVALID
+    assert gemm(mul=7) == INVALID                   # unknown epilogue code
+    assert gemm(mul=2, n=66) == UNSUPPORTED         # gated: N/2 = 33 is not a multiple of 4
     assert gemm(bm=48) == UNSUPPORTED
     assert gemm(dt=0) == UNSUPPORTED                # fp32 has no matrix-core path here
     assert gemm(k=72, astride=72) == UNSUPPORTED    # K must be whole 64-wide steps

@@ -186,3 +186,32 @@ def test_fused_moe_module(ops, dev, grouped):
     layer.pack_weights()
     out2 = layer(x.to(dev), logits.to(dev))
     assert torch.equal(out2, out)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,k,BM,I,K", [
+    (300, 8, 2, 64, 256, 256),
+    (1000, 8, 2, 128, 640, 128),     # I not a multiple of the 128 output columns of a workgroup
+    (40, 4, 2, 256, 96, 64),
+    (77, 4, 1, 32, 20, 64),          # I = 20: row-major only (packed tiles would straddle)
+])
+def test_gated_silu_epilogue_is_bit_identical_to_separate_kernels(ops, dev, dtype, T, E, k, BM, I, K):
+    _, w, ids, s, e, p = _route(T, E, k, BM, T + I)
+    g = gen(I)
+    A = randn((T, K), g, dtype, std=0.5).to(dev)
+    Bw = randn((E, 2 * I, K), g, dtype, std=0.5).to(dev)
+    w, s, e, p = w.to(dev), s.to(dev), e.to(dev), p.to(dev)
+    full = torch.zeros((T, k, 2 * I), dtype=dtype, device=dev)
+    ops.moe_ops.moe_grouped_gemm(A, Bw, full, w, s, e, p, T * k, BM, k, False)
+    want = torch.empty((T * k, I), dtype=dtype, device=dev)
+    ops.activation_ops.silu_and_mul(want, full.view(-1, 2 * I))
+    got = torch.full((T * k, I), 3.0, dtype=dtype, device=dev)
+    ops.moe_ops.moe_grouped_gemm(A, Bw, got, w, s, e, p, T * k, BM, k, False, silu_and_mul=True)
+    assert torch.equal(got, want)
+    if I % 32 == 0:
+        from sarathi_amd.layers import pack_expert_weights
+        packed = pack_expert_weights(Bw)
+        got2 = torch.full((T * k, I), 3.0, dtype=dtype, device=dev)
+        ops.moe_ops.moe_grouped_gemm(A, packed.data, got2, w, s, e, p, T * k, BM, k, False, True,
+                                     2 * I, True)
+        assert torch.equal(got2, want)
