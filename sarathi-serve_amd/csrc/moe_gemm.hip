@@ -91,14 +91,17 @@ struct MoeGemmArgs {
 };
 
 // BM slots per workgroup = WM wave rows x (BM / WM) slots; four wave columns of 64 output columns.
-// WM = 2 (BM = 256, eight waves) halves the number of times a weight tile is pulled out of L2,
-// which is what bounds this kernel once the loads are coalesced.
-// At least two waves per SIMD: with 128 accumulator registers per lane (BM = 128 / 256) that
+// All launches use WM = 1: at BM = 256 a wave then owns a 256 x 64 accumulator tile (256
+// registers, one wave per SIMD), which halves the weight bytes loaded per flop.  That is the
+// fastest shape for row-major weights, whose loads are the bottleneck (830 against 680 TFLOP/s at
+// BM = 128); with packed weights BM = 128 at two waves per SIMD wins (1000 against 850).  WM = 2
+// (eight waves, two of them loading each weight tile) was measured slower than both.
+// Up to BM = 128, at least two waves per SIMD: with 128 accumulator registers per lane that
 // caps the other registers at 128, which the main loop meets anyway (106); without the bound
 // the epilogues that do arithmetic on the accumulators are allocated ~138 and the whole kernel
 // drops to one wave per SIMD (measured: 15 % slower).
 template <int DT, int BM, int WM, int EPI, bool PACKED>
-__global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(2)))
+__global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(BM / WM > 128 ? 1 : 2)))
 void moe_gemm_kernel(MoeGemmArgs g) {
   constexpr bool MUL_WEIGHT = EPI == kEpiMulWeight;
   constexpr bool GATED = EPI == kEpiGatedSilu;
@@ -296,7 +299,7 @@ void moe_gemm_kernel(MoeGemmArgs g) {
 
 template <int DT, int BM>
 static int launch_moe_gemm(const MoeGemmArgs& g, int epilogue, bool packed, hipStream_t st) {
-  constexpr int WM = BM > 128 ? 2 : 1;
+  constexpr int WM = 1;
   const int64_t groups = (g.n_blocks + 7) / 8;
   const int64_t blocks = groups * g.m_blocks * 8;
   if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;

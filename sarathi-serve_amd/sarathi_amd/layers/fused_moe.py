@@ -60,39 +60,47 @@ FUSE_SILU_AND_MUL = True
 CHUNK_SIZE = 64 * 1024     # tokens per pass, as in the reference (fused_moe.py:437)
 
 
-def get_default_config(M: int, E: int, N: int, K: int, topk: int,
-                       dtype: Optional[str] = None) -> Dict[str, int]:
+def get_default_config(M: int, E: int, N: int, K: int, topk: int, dtype: Optional[str] = None,
+                       packed: bool = True) -> Dict[str, int]:
     """Slot-block size for M tokens: the more slots an expert receives, the taller the tile (a
-    taller tile re-uses each weight fragment for more tokens).  BLOCK_SIZE_N / BLOCK_SIZE_K are
-    fixed properties of the kernel and reported for information."""
+    taller tile re-uses each weight fragment for more tokens).  Thresholds from sweeps of the
+    Mixtral-8x7B shape on MI355X (tune_fused_moe.py): with packed weights 256 is never the
+    fastest; with row-major weights, whose loads are the bottleneck, it wins from ~128 slots per
+    expert.  BLOCK_SIZE_N / BLOCK_SIZE_K are fixed properties of the kernel, reported for
+    information."""
     per_expert = M * topk / max(E, 1)
-    # thresholds from a sweep of the Mixtral-8x7B shape on MI355X (tune_fused_moe.py); 256 was
-    # never the fastest
-    block_m = 128 if per_expert >= 48 else 64 if per_expert >= 10 else 32
+    if not packed and per_expert >= 96:
+        block_m = 256
+    else:
+        block_m = 128 if per_expert >= 48 else 64 if per_expert >= 10 else 32
     return {"BLOCK_SIZE_M": block_m, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 64, "GROUP_SIZE_M": 1}
 
 
-def get_config_file_name(E: int, N: int, dtype: Optional[str]) -> str:
-    """Same naming rule as the reference (fused_moe.py:262-265)."""
+def get_config_file_name(E: int, N: int, dtype: Optional[str], packed: bool = True) -> str:
+    """The reference's naming rule (fused_moe.py:262-265), plus a ``,layout=row_major`` selector
+    for tables tuned on un-packed weights."""
     device_name = torch.cuda.get_device_name().replace(" ", "_")
-    dtype_selector = "" if not dtype else f",dtype={dtype}"
-    return f"E={E},N={N},device_name={device_name}{dtype_selector}.json"
+    return f"E={E},N={N},device_name={device_name}{_selectors(dtype, packed)}.json"
+
+
+def _selectors(dtype: Optional[str], packed: bool) -> str:
+    return ("" if not dtype else f",dtype={dtype}") + ("" if packed else ",layout=row_major")
 
 
 CONFIG_DIR = os.path.join(os.path.dirname(os.path.realpath(__file__)), "configs")
 
 
 @functools.lru_cache
-def get_moe_configs(E: int, N: int, dtype: Optional[str]) -> Optional[Dict[int, Any]]:
+def get_moe_configs(E: int, N: int, dtype: Optional[str],
+                    packed: bool = True) -> Optional[Dict[int, Any]]:
     """Tuned slot-block sizes for this (E, N) on this device, as a map batch size -> config, or
     None (reference: fused_moe.py:268-294).  Files are written by ``tune_fused_moe.py``.  MI355X
     boards report different marketing names depending on the driver, so a file named for the
     architecture (``device_name=gfx950``) is tried after the one named for the device."""
-    names = [get_config_file_name(E, N, dtype)]
+    names = [get_config_file_name(E, N, dtype, packed)]
     arch = getattr(torch.cuda.get_device_properties(torch.cuda.current_device()), "gcnArchName", "")
     if arch:
-        dtype_selector = "" if not dtype else f",dtype={dtype}"
-        names.append(f"E={E},N={N},device_name={arch.split(':')[0]}{dtype_selector}.json")
+        names.append(f"E={E},N={N},device_name={arch.split(':')[0]}{_selectors(dtype, packed)}.json")
     for name in names:
         path = os.path.join(CONFIG_DIR, name)
         if os.path.exists(path):
@@ -103,16 +111,17 @@ def get_moe_configs(E: int, N: int, dtype: Optional[str]) -> Optional[Dict[int, 
 
 def try_get_optimal_moe_config(w1_shape: Tuple[int, ...], w2_shape: Tuple[int, ...], top_k: int,
                                M: int, dtype: Optional[str] = None,
-                               override_config: Optional[Dict[str, Any]] = None) -> Dict[str, Any]:
+                               override_config: Optional[Dict[str, Any]] = None,
+                               packed: bool = True) -> Dict[str, Any]:
     """override_config, else the tuned entry closest to M, else the default rule
     (reference: fused_moe.py:321-343)."""
     if override_config:
         return override_config
     E, _, N = w2_shape
-    configs = get_moe_configs(E, N, dtype)
+    configs = get_moe_configs(E, N, dtype, packed)
     if configs:
         return configs[min(configs.keys(), key=lambda x: abs(x - M))]
-    return get_default_config(M, E, N, w1_shape[2], top_k, dtype)
+    return get_default_config(M, E, N, w1_shape[2], top_k, dtype, packed)
 
 
 def invoke_fused_moe_kernel(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor,
@@ -175,7 +184,8 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
         cur_hidden = hidden_states[begin:end]
         cur_ids, cur_w = topk_ids[begin:end], topk_weights[begin:end]
         config = try_get_optimal_moe_config(tuple(w1.shape), tuple(w2.shape), topk, n,
-                                            override_config=override_config)
+                                            override_config=override_config,
+                                            packed=isinstance(w1, PackedExpertWeights))
         c2, c3 = cache2[:n * topk], cache3[:n]
         if _alignment is not None and n == num_tokens and _alignment[3] == config["BLOCK_SIZE_M"]:
             sorted_ids, expert_ids, post_padded = _alignment[:3]
@@ -216,7 +226,8 @@ def fused_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
     elif 0 < num_tokens * topk <= FUSED_ROUTING_MAX_SLOTS:
         # small batches are launch-latency bound: routing and slot sort in one launch
         config = try_get_optimal_moe_config(tuple(w1.shape), tuple(w2.shape), topk, num_tokens,
-                                            override_config=override_config)
+                                            override_config=override_config,
+                                            packed=isinstance(w1, PackedExpertWeights))
         block_m = config["BLOCK_SIZE_M"]
         topk_weights, topk_ids, sorted_ids, expert_ids, post_padded = fused_topk_and_align(
             hidden_states, gating_output, topk, renormalize, block_m)

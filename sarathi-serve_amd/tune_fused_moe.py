@@ -5,8 +5,10 @@ sarathi/model_executor/layers/fused_moe/configs/ and fused_moe.py:262-294).
 
     python sarathi-serve_amd/tune_fused_moe.py --experts 8 --hidden 4096 --intermediate 14336
 
-times ``fused_experts`` (both GEMMs, activation, sort and top-k sum; packed weights) for every block
-size on a grid of batch sizes and keeps the fastest.  One MI355X, synthetic data.
+times ``fused_experts`` (both GEMMs, activation, sort and top-k sum) for every block size on a grid
+of batch sizes and keeps the fastest.  ``--layout row_major`` tunes for the reference's [E, N, K]
+weight tensors (file name suffix ``,layout=row_major``), the default for weights re-tiled with
+``pack_expert_weights``.  One MI355X, synthetic data.
 """
 import argparse
 import json
@@ -28,6 +30,8 @@ def main():
     ap.add_argument("--iters", type=int, default=10)
     ap.add_argument("--out-dir", type=str, default="",
                     help="default: the package's layers/configs directory")
+    ap.add_argument("--layout", choices=["packed", "row_major"], default="packed",
+                    help="expert weight layout the table is for")
     ap.add_argument("--device-name", type=str, default="",
                     help="device_name field of the file name; default: the GPU architecture")
     args = ap.parse_args()
@@ -41,10 +45,10 @@ def main():
     torch.manual_seed(0)
     E, k, H, I = args.experts, args.topk, args.hidden, args.intermediate
     bf = torch.bfloat16
-    w1 = layers.pack_expert_weights(
-        (torch.randn((E, 2 * I, H), device=dev, dtype=torch.float32) * H ** -0.5).to(bf))
-    w2 = layers.pack_expert_weights(
-        (torch.randn((E, H, I), device=dev, dtype=torch.float32) * I ** -0.5).to(bf))
+    w1 = (torch.randn((E, 2 * I, H), device=dev, dtype=torch.float32) * H ** -0.5).to(bf)
+    w2 = (torch.randn((E, H, I), device=dev, dtype=torch.float32) * I ** -0.5).to(bf)
+    if args.layout == "packed":
+        w1, w2 = layers.pack_expert_weights(w1), layers.pack_expert_weights(w2)
 
     def time_ms(fn):
         for _ in range(2):
@@ -79,7 +83,8 @@ def main():
     name = args.device_name or arch
     out_dir = args.out_dir or fm.CONFIG_DIR
     os.makedirs(out_dir, exist_ok=True)
-    path = os.path.join(out_dir, "E=%d,N=%d,device_name=%s.json" % (E, I, name))
+    suffix = "" if args.layout == "packed" else ",layout=row_major"
+    path = os.path.join(out_dir, "E=%d,N=%d,device_name=%s%s.json" % (E, I, name, suffix))
     with open(path, "w") as f:
         json.dump(table, f, indent=4)
         f.write("\n")

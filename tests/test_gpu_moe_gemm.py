@@ -152,6 +152,9 @@ def test_tuned_config_lookup_and_override(ops, dev):
     forced = {"BLOCK_SIZE_M": 32}
     assert layers.try_get_optimal_moe_config(w1_shape, w2_shape, 2, 3000,
                                              override_config=forced) is forced
+    rm = layers.get_moe_configs(8, 14336, None, packed=False)      # table for row-major weights
+    assert rm is not None and rm[4096]["BLOCK_SIZE_M"] == 256
+    assert layers.try_get_optimal_moe_config(w1_shape, w2_shape, 2, 4000, packed=False) == rm[4096]
     assert layers.get_moe_configs(7, 1234, None) is None
     assert layers.try_get_optimal_moe_config((7, 2468, 64), (7, 64, 1234), 2, 512) == \
         layers.get_default_config(512, 7, 1234, 64, 2)
