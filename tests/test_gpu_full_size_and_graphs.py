@@ -161,3 +161,87 @@ def test_chain_and_routing_under_hip_graph_capture(ops, dev):
             assert torch.equal(a, b), "replay %d differs from the eager run" % it
         # unrelated eager work between replays
         _ = (s["gate_up"].float().sum() + gating.sum()).item()
+
+
+def test_kv_append_routing_and_expert_gemm_under_hip_graph_capture(ops, dev):
+    """The rotary + KV-append fusion, the one-launch routing kernel (whose completion counter must be
+    back at zero after every replay) and the grouped GEMM with both epilogues, captured once and
+    replayed with eager work in between; every replay equals the eager run."""
+    import numpy as np
+    from sarathi_amd import layers
+    T, nq, nkv, D, page = 300, 8, 2, 128, 16
+    rng = np.random.default_rng(1)
+    lens = [(True, 200, 260)] + [(False, 1, int(c)) for c in rng.integers(1, 90, size=100)]
+    need = [(t + page - 1) // page for _, _, t in lens]
+    perm = rng.permutation(sum(need))
+    seqs, at = [], 0
+    for (is_p, new, tot), n_pages in zip(lens, need):
+        seqs.append(layers.SequenceSlice(is_p, new, tot, perm[at:at + n_pages].tolist()))
+        at += n_pages
+    meta = layers.build_append_metadata(seqs, page, dev)
+    assert meta.num_total_tokens == T
+    g = gen(11)
+    qkv0 = randn((T, (nq + 2 * nkv) * D), g).to(dev)
+    qkv = qkv0.clone()
+    q, k, v = qkv.split([nq * D, nkv * D, nkv * D], dim=-1)
+    table = cos_sin_cache(4096, D, THETA_LLAMA3, torch.bfloat16).to(dev)
+    positions = meta.append_positions.long()
+    kv_cache = torch.zeros((sum(need), 2, page, nkv, D), dtype=torch.bfloat16, device=dev)
+
+    M, E, topk, B, H, I = 256, 8, 2, 64, 256, 512
+    x = randn((M, H), g).to(dev)
+    w1 = randn((E, 2 * I, H), g, std=H ** -0.5).to(dev)
+    w2 = layers.pack_expert_weights(randn((E, H, I), g, std=I ** -0.5).to(dev))
+    gating = torch.randn((M, E), generator=g, dtype=torch.float32).to(dev)
+    tw = torch.empty((M, topk), dtype=torch.float32, device=dev)
+    ti = torch.empty((M, topk), dtype=torch.int32, device=dev)
+    ts = torch.empty((M, topk), dtype=torch.int32, device=dev)
+    n = M * topk + E * (B - 1)
+    sg = torch.empty((n,), dtype=torch.int32, device=dev)
+    eg = torch.zeros(((n + B - 1) // B,), dtype=torch.int32, device=dev)
+    pg = torch.empty((1,), dtype=torch.int32, device=dev)
+    act = torch.empty((M * topk, I), dtype=torch.bfloat16, device=dev)
+    down = torch.empty((M, topk, H), dtype=torch.bfloat16, device=dev)
+
+    def run_all():
+        ops.kv_cache_ops.rotary_embedding_append_paged_kv(
+            positions, q, k, v, D, table, True, meta.append_batch_indices, meta.append_positions,
+            kv_cache, meta.append_kv_page_indices, meta.append_kv_page_indptr,
+            slot_mapping=meta.slot_mapping)
+        ops.moe_ops.fused_topk_align(tw, ti, ts, gating, True, B, sg, eg, pg, True)
+        ops.moe_ops.moe_grouped_gemm(x, w1, act, tw, sg, eg, pg, M * topk, B, topk, False,
+                                     silu_and_mul=True)
+        ops.moe_ops.moe_grouped_gemm(act, w2.data, down, tw, sg, eg, pg, M * topk, B, 1, True, True, H)
+
+    outs = (qkv, kv_cache, tw, ti, ts, sg, eg, pg, act, down)
+
+    def reset():
+        qkv.copy_(qkv0)
+        for t in (kv_cache, tw, sg, act, down):
+            t.zero_()
+
+    reset()
+    run_all()
+    torch.cuda.synchronize()
+    want = [t.clone() for t in outs]
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        reset()
+        run_all()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    reset()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        run_all()
+    for it in range(4):
+        reset()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(outs, want):
+            assert torch.equal(a, b), "replay %d differs from the eager run" % it
+        _ = (x.float().sum() + gating.sum()).item()
