@@ -189,7 +189,7 @@ static int launch_gelu(void* out, const void* in, int64_t numel, hipStream_t st)
 template <bool FAST>
 static int dispatch_gelu(void* out, const void* in, int64_t T, int64_t d, int dtype,
                          void* stream) {
-  if (!out || !in) return SARATHI_ERR_INVALID_ARG;
+  if (T > 0 && (!out || !in)) return SARATHI_ERR_INVALID_ARG;  // empty tensors have no data
   if (T < 0 || d <= 0) return SARATHI_ERR_INVALID_ARG;
   if (T == 0) return SARATHI_OK;
   hipStream_t st = (hipStream_t)stream;
@@ -208,7 +208,7 @@ extern "C" int sarathi_silu_and_mul(void* out, const void* input, int64_t num_to
                                     int64_t input_row_stride, int64_t out_row_stride, int dtype,
                                     void* stream) {
   using namespace sarathi_hip;
-  if (!out || !input) return SARATHI_ERR_INVALID_ARG;
+  if (num_tokens > 0 && (!out || !input)) return SARATHI_ERR_INVALID_ARG;
   if (num_tokens < 0 || d <= 0 || input_row_stride < 2 * d || out_row_stride < d)
     return SARATHI_ERR_INVALID_ARG;
   if (num_tokens == 0) return SARATHI_OK;

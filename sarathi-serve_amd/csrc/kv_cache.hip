@@ -102,9 +102,9 @@ extern "C" int sarathi_append_paged_kv_cache(
     const int32_t* kv_indptr, const int32_t* slot_mapping, int64_t nnz, int num_kv_heads,
     int head_size, int page_size, int64_t key_stride, int64_t value_stride, int64_t page_stride,
     int64_t entry_stride, int dtype, void* stream) {
-  if (!append_key || !append_value || !k_cache || !v_cache) return SARATHI_ERR_INVALID_ARG;
-  if (!slot_mapping && (!batch_indices || !positions || !kv_indices || !kv_indptr))
-    return SARATHI_ERR_INVALID_ARG;
+  if (nnz > 0 && (!append_key || !append_value || !k_cache || !v_cache ||
+                  (!slot_mapping && (!batch_indices || !positions || !kv_indices || !kv_indptr))))
+    return SARATHI_ERR_INVALID_ARG;  // empty tensors have no data
   const int64_t row = (int64_t)num_kv_heads * head_size;
   if (nnz < 0 || num_kv_heads <= 0 || head_size <= 0 || page_size <= 0 || key_stride < row ||
       value_stride < row || entry_stride < row || page_stride < (int64_t)page_size * entry_stride)

@@ -276,7 +276,10 @@ extern "C" int sarathi_moe_align_block_size(const void* topk_ids, int id_dtype, 
                                             void* workspace, int64_t workspace_bytes,
                                             void* stream) {
   using namespace sarathi_hip;
-  if (!sorted_token_ids || !expert_ids || !num_tokens_post_pad) return SARATHI_ERR_INVALID_ARG;
+  if (!num_tokens_post_pad) return SARATHI_ERR_INVALID_ARG;
+  // empty output buffers (no ids and block_size 1) legitimately come with null pointers
+  if ((sorted_len > 0 && !sorted_token_ids) || (expert_ids_len > 0 && !expert_ids))
+    return SARATHI_ERR_INVALID_ARG;
   if (numel < 0 || (numel > 0 && !topk_ids) || num_experts <= 0 || block_size <= 0 ||
       sorted_len < 0 || expert_ids_len < 0 || workspace_bytes < 0)
     return SARATHI_ERR_INVALID_ARG;

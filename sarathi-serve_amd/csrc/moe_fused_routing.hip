@@ -81,8 +81,10 @@ extern "C" int sarathi_fused_topk_align(float* topk_weights, int32_t* topk_indic
                                         int32_t* num_tokens_post_pad, int fill_pad,
                                         uint32_t* counter, void* stream) {
   using namespace sarathi_hip;
-  if (!topk_weights || !topk_indices || !token_expert_indices || !gating_output ||
-      !sorted_token_ids || !expert_ids || !num_tokens_post_pad)
+  if (!num_tokens_post_pad || (sorted_len > 0 && !sorted_token_ids) ||
+      (expert_ids_len > 0 && !expert_ids))
+    return SARATHI_ERR_INVALID_ARG;
+  if (num_tokens > 0 && (!topk_weights || !topk_indices || !token_expert_indices || !gating_output))
     return SARATHI_ERR_INVALID_ARG;
   if (num_tokens < 0 || num_experts <= 0 || topk <= 0 || topk > num_experts || block_size <= 0 ||
       sorted_len < 0 || expert_ids_len < 0)
@@ -100,6 +102,7 @@ extern "C" int sarathi_fused_topk_align(float* topk_weights, int32_t* topk_indic
                        (E & (E - 1)) == 0 && E <= 256 &&
                        (reinterpret_cast<uintptr_t>(gating_output) & (E < 4 ? E * 4 - 1 : 15)) == 0;
   if (!fusable) {
+    // (zero tokens: topk_softmax is a no-op and the sort still writes num_tokens_post_pad = 0)
     int rc = sarathi_topk_softmax(topk_weights, topk_indices, token_expert_indices, gating_output,
                                   num_tokens, num_experts, topk, renormalize, stream);
     if (rc != SARATHI_OK) return rc;

@@ -151,8 +151,8 @@ extern "C" int sarathi_topk_softmax(float* topk_weights, int32_t* topk_indices,
                                     int64_t num_tokens, int num_experts, int topk,
                                     int renormalize, void* stream) {
   using namespace sarathi_hip;
-  if (!topk_weights || !topk_indices || !token_expert_indices || !gating_output)
-    return SARATHI_ERR_INVALID_ARG;
+  if (num_tokens > 0 && (!topk_weights || !topk_indices || !token_expert_indices || !gating_output))
+    return SARATHI_ERR_INVALID_ARG;  // empty tensors have no data
   if (num_tokens < 0 || num_experts <= 0 || topk <= 0 || topk > num_experts)
     return SARATHI_ERR_INVALID_ARG;
   if (num_experts > SARATHI_MOE_MAX_EXPERTS) return SARATHI_ERR_UNSUPPORTED;
@@ -194,7 +194,8 @@ extern "C" int sarathi_grouped_topk(float* topk_weights, int32_t* topk_indices,
                                     int num_experts, int topk, int num_expert_group,
                                     int topk_group, int renormalize, void* stream) {
   using namespace sarathi_hip;
-  if (!topk_weights || !topk_indices || !gating_output) return SARATHI_ERR_INVALID_ARG;
+  if (num_tokens > 0 && (!topk_weights || !topk_indices || !gating_output))
+    return SARATHI_ERR_INVALID_ARG;
   if (num_tokens < 0 || num_experts <= 0 || topk <= 0 || topk > num_experts ||
       num_expert_group <= 0 || topk_group <= 0 || topk_group > num_expert_group ||
       num_experts % num_expert_group != 0)

@@ -166,7 +166,7 @@ static int launch_rms(void* out, void* in, const void* w, float eps, int64_t T, 
 template <bool FUSED>
 static int dispatch_rms(void* out, void* in, const void* w, float eps, int64_t T, int64_t H,
                         int64_t out_stride, int64_t in_stride, int dtype, void* stream) {
-  if (!out || !in || !w) return SARATHI_ERR_INVALID_ARG;
+  if (T > 0 && (!out || !in || !w)) return SARATHI_ERR_INVALID_ARG;  // empty tensors have no data
   if (T < 0 || H <= 0 || out_stride < H || in_stride < H) return SARATHI_ERR_INVALID_ARG;
   if (H > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
   if (T == 0) return SARATHI_OK;

@@ -417,7 +417,8 @@ extern "C" int sarathi_rotary_embedding(const int64_t* positions, void* query, v
                                         int rot_dim, int64_t query_stride, int64_t key_stride,
                                         int is_neox, int dtype, void* stream) {
   using namespace sarathi_hip;
-  if (!positions || !query || !key || !cos_sin_cache) return SARATHI_ERR_INVALID_ARG;
+  if (num_tokens > 0 && (!positions || !query || !key || !cos_sin_cache))
+    return SARATHI_ERR_INVALID_ARG;  // empty tensors have no data
   if (num_tokens < 0 || num_heads <= 0 || num_kv_heads < 0 || head_size <= 0 || rot_dim <= 0 ||
       (rot_dim & 1) || rot_dim > head_size)
     return SARATHI_ERR_INVALID_ARG;
@@ -447,9 +448,11 @@ extern "C" int sarathi_rotary_embedding_append_paged_kv(
     int64_t page_stride, int64_t entry_stride, int is_neox, int write_key, int dtype,
     void* stream) {
   using namespace sarathi_hip;
-  if (!positions || !query || !key || !value || !cos_sin_cache || !k_cache || !v_cache)
+  if (num_tokens > 0 && (!positions || !query || !key || !value || !cos_sin_cache))
     return SARATHI_ERR_INVALID_ARG;
-  if (!slot_mapping && (!batch_indices || !append_positions || !kv_indices || !kv_indptr))
+  if (num_append_tokens > 0 &&
+      (!k_cache || !v_cache ||
+       (!slot_mapping && (!batch_indices || !append_positions || !kv_indices || !kv_indptr))))
     return SARATHI_ERR_INVALID_ARG;
   if (num_tokens < 0 || num_append_tokens < 0 || num_append_tokens > num_tokens ||
       num_heads <= 0 || num_kv_heads <= 0 || head_size <= 0 || rot_dim <= 0 || (rot_dim & 1) ||

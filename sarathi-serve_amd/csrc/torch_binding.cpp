@@ -1,14 +1,16 @@
 // PyTorch-ROCm front end of the op library: a pybind11 module whose functions
 // have the names and positional signatures of the reference's four extension
 // modules (csrc/layernorm.cpp:9, csrc/activation.cpp:15-27, csrc/pos_encoding.cpp:11,
-// csrc/moe.cpp:19-27), plus fused_add_rms_norm and two fused MoE variants.
+// csrc/moe.cpp:19-27), plus the entries the reference does not have: fused_add_rms_norm, the
+// fused MoE routing variants, grouped_topk, the grouped expert GEMM and the paged KV-cache ops.
 //
 // This layer only (a) checks what the reference leaves unchecked: device, dtype,
 // rank, inner contiguity; (b) makes the tensors' device current and looks up
 // torch's current HIP stream for it; (c) forwards raw pointers, sizes and
 // strides to the C ABI of include/sarathi_ops.h and turns a non-zero status
 // into a RuntimeError.  It never copies or synchronises, and allocates only the scratch
-// tensor that moe_align_block_size uses for inputs above 16 K ids.
+// tensor that moe_align_block_size uses for inputs above 16 K ids and, once per (device, stream),
+// the four-byte completion counter of fused_topk_align.
 #include <c10/hip/HIPStream.h>
 #include <hip/hip_runtime_api.h>
 #include <torch/extension.h>
@@ -109,7 +111,8 @@ void fused_add_rms_norm(torch::Tensor& input, torch::Tensor& residual, torch::Te
   TORCH_CHECK(weight.dim() == 1 && weight.size(0) == input.size(1) && weight.is_contiguous(), op,
               ": weight must be a contiguous [hidden] vector");
   TORCH_CHECK(input.stride(1) == 1 && residual.stride(1) == 1, op, ": rows must be contiguous");
-  TORCH_CHECK(input.data_ptr() != residual.data_ptr(), op, ": input and residual must not alias");
+  TORCH_CHECK(input.numel() == 0 || input.data_ptr() != residual.data_ptr(), op,
+              ": input and residual must not alias");
   LaunchScope scope(input);
   raise_on(sarathi_fused_add_rms_norm(input.data_ptr(), residual.data_ptr(), weight.data_ptr(),
                                       (float)epsilon, input.size(0), input.size(1),

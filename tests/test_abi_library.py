@@ -63,6 +63,8 @@ def test_argument_validation_without_gpu(lib):
     assert rms(p, p, p, f32(1e-5), i64(1), i64(8), i64(4), i64(8), ci(2), null) == INVALID  # stride < H
     assert rms(p, p, p, f32(1e-5), i64(1), i64(8), i64(8), i64(8), ci(7), null) == UNSUPPORTED
     assert rms(p, p, p, f32(1e-5), i64(0), i64(8), i64(8), i64(8), ci(2), null) == OK
+    # an empty batch comes with null data pointers (an empty tensor owns no memory): still a no-op
+    assert rms(null, null, p, f32(1e-5), i64(0), i64(8), i64(8), i64(8), ci(2), null) == OK
     fused = lib.sarathi_fused_add_rms_norm
     assert fused(p, null, p, f32(1e-5), i64(1), i64(8), i64(8), i64(8), ci(2), null) == INVALID
     assert fused(p, p, p, f32(1e-5), i64(0), i64(8), i64(8), i64(8), ci(2), null) == OK
@@ -71,6 +73,7 @@ def test_argument_validation_without_gpu(lib):
     assert silu(p, p, i64(1), i64(8), i64(8), i64(8), ci(2), null) == INVALID      # stride < 2d
     assert silu(p, p, i64(1), i64(8), i64(16), i64(8), ci(9), null) == UNSUPPORTED
     assert silu(p, p, i64(0), i64(8), i64(16), i64(8), ci(2), null) == OK
+    assert silu(null, null, i64(0), i64(8), i64(16), i64(8), ci(2), null) == OK
     for gelu in (lib.sarathi_gelu_new, lib.sarathi_gelu_fast):
         assert gelu(null, p, i64(1), i64(8), ci(2), null) == INVALID
         assert gelu(p, p, i64(1), i64(0), ci(2), null) == INVALID
@@ -91,6 +94,7 @@ def test_argument_validation_without_gpu(lib):
     assert topk(p, p, p, p, i64(1), ci(0), ci(1), ci(0), null) == INVALID
     assert topk(p, p, p, p, i64(1), ci(2048), ci(1), ci(0), null) == UNSUPPORTED
     assert topk(p, p, p, p, i64(0), ci(8), ci(2), ci(0), null) == OK
+    assert topk(null, null, null, null, i64(0), ci(8), ci(2), ci(0), null) == OK
     align = lib.sarathi_moe_align_block_size
     ws = (null, i64(0), null)      # workspace, workspace_bytes, stream
     assert align(p, ci(3), i64(4), ci(8), ci(4), null, i64(64), p, i64(16), p, ci(0), *ws) == INVALID
@@ -99,6 +103,8 @@ def test_argument_validation_without_gpu(lib):
     assert align(p, ci(3), i64(4), ci(8), ci(4), p, i64(64), p, i64(1), p, ci(0), *ws) == INVALID  # expert_ids too short
     assert align(p, ci(3), i64(4), ci(4096), ci(4), p, i64(64), p, i64(16), p, ci(0), *ws) == UNSUPPORTED
     assert align(p, ci(11), i64(4), ci(8), ci(4), p, i64(64), p, i64(16), p, ci(0), *ws) == UNSUPPORTED
+    # no ids and block_size 1: the output buffers are empty and may be null; post_pad is written
+    assert align(null, ci(3), i64(0), ci(8), ci(1), null, i64(0), null, i64(0), null, ci(0), *ws) == INVALID
     wsb = lib.sarathi_moe_align_workspace_bytes
     wsb.restype = ctypes.c_int64
     assert wsb(i64(8192), ci(8)) == 0                       # small inputs: single workgroup

@@ -229,3 +229,35 @@ def test_rope_position_zero_is_identity_and_norm_preserved(ops, dev):
     n0 = q.view(T, nq, 2, D // 2).pow(2).sum(2)
     n1 = gq.cpu().view(T, nq, 2, D // 2).pow(2).sum(2)
     assert torch.allclose(n0, n1, rtol=1e-5, atol=1e-6)              # rotations keep |(x, y)|
+
+
+def test_empty_batch_is_a_no_op_everywhere(ops, dev):
+    """Zero tokens: every op returns without touching anything (empty tensors own no memory, so
+    the C ABI sees null data pointers); the slot sort still reports zero padded tokens."""
+    bf = torch.bfloat16
+    e = lambda *shape, dt=bf: torch.empty(shape, dtype=dt, device=dev)  # noqa: E731
+    w = torch.ones(64, dtype=bf, device=dev)
+    ops.layernorm_ops.rms_norm(e(0, 64), e(0, 64), w, 1e-5)
+    ops.layernorm_ops.fused_add_rms_norm(e(0, 64), e(0, 64), w, 1e-5)
+    ops.activation_ops.silu_and_mul(e(0, 32), e(0, 64))
+    ops.activation_ops.gelu_new(e(0, 64), e(0, 64))
+    ops.activation_ops.gelu_fast(e(0, 64), e(0, 64))
+    table = torch.zeros((16, 32), dtype=bf, device=dev)
+    ops.pos_encoding_ops.rotary_embedding(e(0, dt=torch.int64), e(0, 128), e(0, 64), 32, table, True)
+    i32 = torch.int32
+    ops.moe_ops.topk_softmax(e(0, 2, dt=torch.float32), e(0, 2, dt=i32), e(0, 2, dt=i32),
+                             e(0, 8, dt=torch.float32))
+    post = torch.full((1,), -1, dtype=i32, device=dev)
+    ops.moe_ops.moe_align_block_size(e(0, 2, dt=i32), 8, 1, e(0, dt=i32), e(0, dt=i32), post)
+    assert int(post.item()) == 0
+    post.fill_(-1)
+    sorted_ids = torch.full((8 * 15,), -7, dtype=i32, device=dev)
+    ops.moe_ops.fused_topk_align(e(0, 2, dt=torch.float32), e(0, 2, dt=i32), e(0, 2, dt=i32),
+                                 e(0, 8, dt=torch.float32), True, 16, sorted_ids,
+                                 e(8, dt=i32), post, False)
+    assert int(post.item()) == 0 and bool((sorted_ids == -7).all())
+    cache = torch.zeros((4, 2, 16, 2, 32), dtype=bf, device=dev)
+    ops.kv_cache_ops.append_paged_kv_cache(e(0, 2, 32), e(0, 2, 32), e(0, dt=i32), e(0, dt=i32), cache,
+                                           e(0, dt=i32), torch.zeros(1, dtype=i32, device=dev))
+    assert not bool(cache.any())
+    torch.cuda.synchronize()
