@@ -60,6 +60,19 @@ BYTES["rotary_embedding_append_paged_kv"] = (2 * T * NQ * D + 4 * T * NKV * D) *
 BYTES["append_paged_kv_cache (slot mapping)"] = 4 * T * NKV * D * BF16 + T * 4
 BYTES["rotary_embedding_append_paged_kv (slot mapping)"] = \
     BYTES["rotary_embedding_append_paged_kv"] - T * 12
+# the reference's operation-metric names for the places these ops run at
+# (sarathi/metrics/constants.py:9-34), so that reports line up with its own per-op timers
+REFERENCE_LABELS = {
+    "fused_add_rms_norm": "input_layernorm / post_attention_layernorm",
+    "rms_norm": "input_layernorm / post_attention_layernorm",
+    "rotary_embedding": "attn_rope",
+    "silu_and_mul": "mlp_activation",
+    "append_paged_kv_cache": "attn_kv_cache_save",
+    "rotary_embedding_append_paged_kv": "attn_rope + attn_kv_cache_save",
+    "topk_softmax": "moe_gating",
+    "moe_align_block_size": "moe_linear (slot sort)",
+    "fused_topk_align": "moe_gating + moe_linear (slot sort)",
+}
 MOE_T, MOE_E, MOE_K, MOE_B = 4096, 8, 2, 64
 BYTES["topk_softmax"] = MOE_T * MOE_E * 4 + 3 * MOE_T * MOE_K * 4
 _moe_sorted = MOE_T * MOE_K + MOE_E * (MOE_B - 1)
@@ -276,6 +289,8 @@ def main():
     per_op = {}
     for name, (args_ring, fn) in ops_table.items():
         row = {"bytes": BYTES[name]}
+        if name.split(" ")[0] in REFERENCE_LABELS:
+            row["reference_label"] = REFERENCE_LABELS[name.split(" ")[0]]
         latency_bound = name in ("topk_softmax", "moe_align_block_size", "fused_topk_align")
         for label in ("cold", "warm"):
             if latency_bound and label == "cold":
