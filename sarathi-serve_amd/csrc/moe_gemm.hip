@@ -215,6 +215,8 @@ void moe_gemm_kernel(MoeGemmArgs g) {
   stage(0, anext);
   __syncthreads();
 
+  // (Meeting the other waves one sub-step earlier, so that the next K-step's first operand read
+  // is already in flight under this K-step's last MFMAs, was measured and is 1-4 % slower.)
   // The loop body is branch-free so that the scheduler can keep loads, LDS reads and MFMAs
   // interleaved: the last step simply loads the wrapped-around "next" K-step again (issued,
   // never used), and the token operands of sub-step s + 1 are read from LDS before the MFMAs
