@@ -98,23 +98,23 @@ struct MoeGemmArgs {
   int32_t m_blocks, n_blocks;
 };
 
-// BM slots per workgroup = WM wave rows x (BM / WM) slots; four wave columns of 64 output columns.
-// All launches use WM = 1: at BM = 256 a wave then owns a 256 x 64 accumulator tile (256
-// registers, one wave per SIMD), which halves the weight bytes loaded per flop.  That is the
-// fastest shape for row-major weights, whose loads are the bottleneck (830 against 680 TFLOP/s at
-// BM = 128); with packed weights BM = 128 at two waves per SIMD wins (1000 against 850).  WM = 2
-// (eight waves, two of them loading each weight tile) was measured slower than both.
+// A workgroup is four waves side by side, each owning all BM slots x 64 output columns.  At
+// BM = 256 a wave holds a 256 x 64 accumulator tile (256 registers, one wave per SIMD), which
+// halves the weight bytes loaded per flop: the fastest shape for row-major weights, whose loads
+// are the bottleneck (880 against 725 TFLOP/s at BM = 128); with packed weights BM = 128 at two
+// waves per SIMD wins (1060 against 910).  Eight-wave workgroups with two wave rows sharing each
+// weight tile through the L1 were measured slower than both.
 // Up to BM = 128, at least two waves per SIMD: with 128 accumulator registers per lane that
 // caps the other registers at 128, which the main loop meets anyway (106); without the bound
 // the epilogues that do arithmetic on the accumulators are allocated ~138 and the whole kernel
 // drops to one wave per SIMD (measured: 15 % slower).
-template <int DT, int BM, int WM, int EPI, bool PACKED>
-__global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(BM / WM > 128 ? 1 : 2)))
+template <int DT, int BM, int EPI, bool PACKED>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM > 128 ? 1 : 2)))
 void moe_gemm_kernel(MoeGemmArgs g) {
   constexpr bool MUL_WEIGHT = EPI == kEpiMulWeight;
   constexpr bool GATED = EPI == kEpiGatedSilu;
-  constexpr int THREADS = 256 * WM;
-  constexpr int MT = BM / WM / 32;     // token tiles per wave
+  constexpr int THREADS = 256;
+  constexpr int MT = BM / 32;          // token tiles per wave
   constexpr int NT = kGemmWaveN / 32;  // weight tiles per wave
   constexpr int SUB = kGemmBK / 16;    // MFMA sub-steps per K-step
   constexpr int ROWS_PER_PASS = THREADS / 8;
@@ -131,8 +131,7 @@ void moe_gemm_kernel(MoeGemmArgs g) {
   const int expert = g.expert_ids[pid_m];
 
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = (tid >> 6) & 3;          // wave column: output columns [64 wave, 64 wave + 64)
-  const int row0 = (tid >> 8) * (BM / WM);  // wave row: first slot of this wave inside the block
+  const int wave = tid >> 6;  // output columns [64 wave, 64 wave + 64)
   const int l32 = lane & 31, grp = lane >> 5;
 
   // ---- weights: buffer resource over the expert's matrix; rows >= N read as zero
@@ -224,7 +223,7 @@ void moe_gemm_kernel(MoeGemmArgs g) {
   auto read_tokens = [&](int buf, int s, u32x4 (&tokv)[MT]) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      const int r = row0 + mt * 32 + l32;
+      const int r = mt * 32 + l32;
       tokv[mt] = tok_lds[buf][r * 8 + lds_slot(r, 2 * s + grp)];
     }
   };
@@ -258,7 +257,7 @@ void moe_gemm_kernel(MoeGemmArgs g) {
   // ---- epilogue: lane holds, per accumulator quad, 4 consecutive columns of one token
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const int slot_index = pid_m * BM + row0 + mt * 32 + l32;
+    const int slot_index = pid_m * BM + mt * 32 + l32;
     const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
     if (sid >= g.num_valid) continue;
     float scale = 1.f;
@@ -309,13 +308,12 @@ void moe_gemm_kernel(MoeGemmArgs g) {
 
 template <int DT, int BM>
 static int launch_moe_gemm(const MoeGemmArgs& g, int epilogue, bool packed, hipStream_t st) {
-  constexpr int WM = 1;
   const int64_t groups = (g.n_blocks + 7) / 8;
   const int64_t blocks = groups * g.m_blocks * 8;
   if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
-  const dim3 grid((unsigned)blocks), block(256 * WM);
+  const dim3 grid((unsigned)blocks), block(256);
 #define SK_LAUNCH(EP, PK) \
-  hipLaunchKernelGGL((moe_gemm_kernel<DT, BM, WM, EP, PK>), grid, block, 0, st, g)
+  hipLaunchKernelGGL((moe_gemm_kernel<DT, BM, EP, PK>), grid, block, 0, st, g)
   if (epilogue == kEpiMulWeight) {
     if (packed) SK_LAUNCH(kEpiMulWeight, true); else SK_LAUNCH(kEpiMulWeight, false);
   } else if (epilogue == kEpiGatedSilu) {
