@@ -25,6 +25,10 @@ def main():
     ap.add_argument("--intermediate", type=int, default=14336)
     ap.add_argument("--block-m", type=int, default=0, help="0 = the wrapper's own choice")
     ap.add_argument("--iters", type=int, default=20)
+    ap.add_argument("--data", choices=["random", "constant"], default="random",
+                    help="constant: every activation and weight holds the same value, which toggles "
+                         "far fewer bits per operation; shows how much of the gap to the nominal "
+                         "peak is the clock the chip sustains under switching power")
     args = ap.parse_args()
 
     import torch
@@ -40,6 +44,10 @@ def main():
     w1 = (torch.randn((E, 2 * I, H), device=dev, dtype=torch.float32) * H ** -0.5).to(bf)
     w2 = (torch.randn((E, H, I), device=dev, dtype=torch.float32) * I ** -0.5).to(bf)
     gating = torch.randn((T, E), device=dev, dtype=torch.float32)
+    if args.data == "constant":
+        x.fill_(0.0078125)
+        w1.fill_(0.0078125)
+        w2.fill_(0.0078125)
     config = dict(get_default_config(T, E, I, H, k))
     if args.block_m:
         config["BLOCK_SIZE_M"] = args.block_m
@@ -99,7 +107,7 @@ def main():
     out = {
         "metric": "grouped expert GEMM TFLOP/s (Mixtral-8x7B MoE layer shape)",
         "config": {"tokens": T, "experts": E, "topk": k, "hidden": H, "intermediate": I,
-                   "dtype": "bf16", "block_m": bm, "device": torch.cuda.get_device_name(0)},
+                   "dtype": "bf16", "block_m": bm, "data": args.data, "device": torch.cuda.get_device_name(0)},
         "weights": res,
         "weight_bytes": (E * 2 * I * H + E * H * I) * 2,
     }
