@@ -518,16 +518,17 @@ void grouped_topk(torch::Tensor& topk_weights, torch::Tensor& topk_indices,
 }
 
 // One zeroed uint32 per (device, stream): the completion counter of the fused routing kernel.
-// Allocated on first use and kept for the life of the process.
+// Allocated on first use and kept for the life of the process; the map is deliberately never
+// destroyed, so no tensor is released after the runtime has shut down at process exit.
 uint32_t* routing_counter(int dev, void* stream) {
   static std::mutex mu;
-  static std::map<std::pair<int, void*>, torch::Tensor> counters;
+  static auto* counters = new std::map<std::pair<int, void*>, torch::Tensor>();
   std::lock_guard<std::mutex> lock(mu);
   auto key = std::make_pair(dev, stream);
-  auto it = counters.find(key);
-  if (it == counters.end()) {
+  auto it = counters->find(key);
+  if (it == counters->end()) {
     auto t = torch::zeros({1}, torch::TensorOptions().dtype(torch::kInt32).device(torch::kCUDA, dev));
-    it = counters.emplace(key, t).first;
+    it = counters->emplace(key, t).first;
   }
   return reinterpret_cast<uint32_t*>(it->second.data_ptr<int32_t>());
 }
