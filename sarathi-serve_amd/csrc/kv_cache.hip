@@ -152,9 +152,9 @@ extern "C" int sarathi_append_paged_kv_cache(
 extern "C" int sarathi_get_seq_lens(const int32_t* kv_indptr, const int32_t* kv_last_page_len,
                                     int32_t* seq_lens, int64_t num_seqs, int page_size,
                                     void* stream) {
-  if (!kv_indptr || !kv_last_page_len || !seq_lens || num_seqs < 0 || page_size <= 0)
-    return SARATHI_ERR_INVALID_ARG;
-  if (num_seqs == 0) return SARATHI_OK;
+  if (num_seqs < 0 || page_size <= 0) return SARATHI_ERR_INVALID_ARG;
+  if (num_seqs == 0) return SARATHI_OK;  // empty tensors have no data: pointers may be null
+  if (!kv_indptr || !kv_last_page_len || !seq_lens) return SARATHI_ERR_INVALID_ARG;
   if (num_seqs > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(kv_seq_lens_kernel, dim3((unsigned)((num_seqs + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, kv_indptr, kv_last_page_len, seq_lens, num_seqs,
@@ -166,9 +166,9 @@ extern "C" int sarathi_get_batch_indices_positions(const int32_t* append_indptr,
                                                    const int32_t* seq_lens, int32_t* batch_indices,
                                                    int32_t* positions, int64_t num_seqs,
                                                    int64_t nnz, void* stream) {
-  if (!append_indptr || !seq_lens || !batch_indices || !positions || num_seqs < 0 || nnz < 0)
-    return SARATHI_ERR_INVALID_ARG;
+  if (num_seqs < 0 || nnz < 0) return SARATHI_ERR_INVALID_ARG;
   if (num_seqs == 0 || nnz == 0) return SARATHI_OK;
+  if (!append_indptr || !seq_lens || !batch_indices || !positions) return SARATHI_ERR_INVALID_ARG;
   if (nnz > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(kv_batch_positions_kernel, dim3((unsigned)((nnz + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, append_indptr, seq_lens, batch_indices, positions,
@@ -180,10 +180,10 @@ extern "C" int sarathi_get_kv_slot_mapping(const int32_t* batch_indices, const i
                                            const int32_t* kv_indices, const int32_t* kv_indptr,
                                            int32_t* slot_mapping, int64_t nnz, int page_size,
                                            void* stream) {
-  if (!batch_indices || !positions || !kv_indices || !kv_indptr || !slot_mapping || nnz < 0 ||
-      page_size <= 0)
-    return SARATHI_ERR_INVALID_ARG;
+  if (nnz < 0 || page_size <= 0) return SARATHI_ERR_INVALID_ARG;
   if (nnz == 0) return SARATHI_OK;
+  if (!batch_indices || !positions || !kv_indices || !kv_indptr || !slot_mapping)
+    return SARATHI_ERR_INVALID_ARG;
   if (nnz > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(kv_slot_mapping_kernel, dim3((unsigned)((nnz + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, batch_indices, positions, kv_indices, kv_indptr,

@@ -68,5 +68,6 @@ def assert_close_dtype(got, want, atol=1e-2, rtol=1e-2, max_ulps=2, max_mismatch
         ulp = torch.maximum(ulp_of(got), ulp_of(want))[fin]
         ulps = (diff / ulp)[bad].max().item()
         assert ulps <= max_ulps + 1e-3, "max error %.2f ulp" % ulps
-    assert frac <= max_mismatch_frac, "mismatching fraction %.3g" % frac
+    # the fraction is a statistical bound: a tiny tensor may hold a couple of one-ulp flips
+    assert frac <= max(max_mismatch_frac, 2.0 / diff.numel()), "mismatching fraction %.3g" % frac
     return frac

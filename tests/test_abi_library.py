@@ -173,6 +173,8 @@ def test_kv_cache_and_gemm_argument_validation_without_gpu(lib):
     assert lib.sarathi_get_batch_indices_positions(p, p, null, p, i64(1), i64(1), null) == INVALID
     assert lib.sarathi_get_batch_indices_positions(p, p, p, p, i64(0), i64(0), null) == OK
     assert lib.sarathi_get_kv_slot_mapping(p, p, p, p, null, i64(1), ci(4), null) == INVALID
+    assert lib.sarathi_get_kv_slot_mapping(null, null, p, p, null, i64(0), ci(4), null) == OK
+    assert lib.sarathi_get_batch_indices_positions(p, p, null, null, i64(1), i64(0), null) == OK
     assert lib.sarathi_get_kv_slot_mapping(p, p, p, p, p, i64(0), ci(4), null) == OK
 
     def fused(**kw):

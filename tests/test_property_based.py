@@ -2,6 +2,8 @@
 list of cases.  The CPU half exercises the oracle's invariants; the GPU half (marked ``gpu``)
 compares the HIP ops with the oracle on the drawn inputs, bit-exact wherever the op is integer /
 byte / index work or pure rounding-defined arithmetic."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -11,8 +13,10 @@ from hypothesis import strategies as st
 from helpers import assert_close_dtype, cos_sin_cache, gen, randn
 from oracle import c_oracle, paged_kv
 
-CPU = settings(max_examples=60, deadline=None, suppress_health_check=list(HealthCheck))
-GPU = settings(max_examples=40, deadline=None, suppress_health_check=list(HealthCheck))
+# SARATHI_TEST_EXAMPLES scales the number of drawn cases for an occasional longer soak
+_SCALE = max(1, int(os.environ.get("SARATHI_TEST_EXAMPLES", "1")))
+CPU = settings(max_examples=60 * _SCALE, deadline=None, suppress_health_check=list(HealthCheck))
+GPU = settings(max_examples=40 * _SCALE, deadline=None, suppress_health_check=list(HealthCheck))
 
 
 def _align_oracle(ids, E, B):
@@ -196,3 +200,114 @@ def test_gpu_topk_softmax_any_expert_count(ops, dev, E, k, T, renorm, seed):
                                                                              gating.to(dev))
     assert torch.equal(gi.cpu(), wi) and torch.equal(gs.cpu(), ws)
     assert torch.allclose(gw.cpu(), ww, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.gpu
+@GPU
+@given(page=st.sampled_from([1, 4, 16, 32]), nkv=st.integers(1, 4),
+       D=st.sampled_from([8, 24, 64, 128, 6]), dt=st.sampled_from(DTYPES), neox=st.booleans(),
+       write_key=st.booleans(), use_slots=st.booleans(), pad=st.integers(0, 3), data=st.data())
+def test_gpu_kv_append_and_fusion_any_layout(ops, dev, page, nkv, D, dt, neox, write_key, use_slots,
+                                             pad, data):
+    """Stand-alone append against the numpy oracle (byte-exact); the rotary + append fusion against
+    the two separate GPU ops (byte-exact on cache, query, key and value)."""
+    R = data.draw(st.integers(1, 5))
+    before = [data.draw(st.integers(0, 50)) for _ in range(R)]
+    new = [data.draw(st.integers(0, 12)) for _ in range(R)]
+    seed = data.draw(st.integers(0, 10 ** 6))
+    totals = [a + b for a, b in zip(before, new)]
+    need = [(t + page - 1) // page for t in totals]
+    rng = np.random.default_rng(seed)
+    pages = sum(need) + 1
+    kv_indices = rng.permutation(pages)[:sum(need)].astype(np.int32)
+    kv_indptr = np.concatenate([[0], np.cumsum(need)]).astype(np.int32)
+    last = np.array([(t % page) or page if t else 0 for t in totals], dtype=np.int32)
+    indptr = np.concatenate([[0], np.cumsum(new)]).astype(np.int32)
+    n = int(indptr[-1])
+    T = n + pad
+    if T == 0:
+        return
+    nq = 2
+    g = gen(seed)
+    t = lambda a: torch.from_numpy(a).to(dev)  # noqa: E731
+    seq_lens = ops.kv_cache_ops.get_seq_lens(t(kv_indptr), t(last), page)
+    assert seq_lens.cpu().tolist() == totals
+    b, ap = ops.kv_cache_ops.get_batch_indices_positions(t(indptr), seq_lens, n)
+    wb, wap = paged_kv.get_batch_indices_positions(indptr, np.array(totals), n)
+    assert b.cpu().tolist() == wb.tolist() and ap.cpu().tolist() == wap.tolist()
+    slots = ops.kv_cache_ops.get_kv_slot_mapping(b, ap, t(kv_indices), t(kv_indptr), page) \
+        if use_slots else None
+
+    qkv = randn((T, (nq + 2 * nkv) * D), g, dt)
+    cache0 = randn((pages, 2, page, nkv, D), g, dt)
+    table = cos_sin_cache(64, D, 10000.0, dt).to(dev)
+    pos = torch.randint(0, 64, (T,), generator=g, dtype=torch.int64).to(dev)
+    split = [nq * D, nkv * D, nkv * D]
+    bits = torch.int16 if dt != torch.float32 else torch.int32
+
+    # separate ops: rotary in place, then append the first n rows
+    sep = qkv.to(dev)
+    sq, sk, sv = sep.split(split, dim=-1)
+    ops.pos_encoding_ops.rotary_embedding(pos, sq, sk, D, table, neox)
+    cache_sep = cache0.to(dev)
+    ops.kv_cache_ops.append_paged_kv_cache(sk[:n], sv[:n], b, ap, cache_sep, t(kv_indices),
+                                           t(kv_indptr), slot_mapping=slots)
+    want = cache0.clone().view(bits).numpy()
+    paged_kv.append_paged_kv_cache(sk[:n].cpu().contiguous().view(bits).numpy().reshape(n, nkv, D),
+                                   sv[:n].cpu().contiguous().view(bits).numpy().reshape(n, nkv, D),
+                                   wb, wap, want[:, 0], want[:, 1], kv_indices, kv_indptr)
+    assert np.array_equal(cache_sep.cpu().view(bits).numpy(), want)
+
+    fused = qkv.to(dev)
+    fq, fk, fv = fused.split(split, dim=-1)
+    cache_fused = cache0.to(dev)
+    ops.kv_cache_ops.rotary_embedding_append_paged_kv(pos, fq, fk, fv, D, table, neox, b, ap,
+                                                      cache_fused, t(kv_indices), t(kv_indptr),
+                                                      num_append_tokens=n, write_key=write_key,
+                                                      slot_mapping=slots)
+    assert torch.equal(cache_fused.view(bits), cache_sep.view(bits))
+    assert torch.equal(fq.contiguous().view(bits), sq.contiguous().view(bits))
+    assert torch.equal(fv.contiguous().view(bits), sv.contiguous().view(bits))
+    assert torch.equal(fk[n:].contiguous().view(bits), sk[n:].contiguous().view(bits))
+    key_want = sk[:n] if write_key else qkv.to(dev).split(split, dim=-1)[1][:n]
+    assert torch.equal(fk[:n].contiguous().view(bits), key_want.contiguous().view(bits))
+
+
+@pytest.mark.gpu
+@GPU
+@given(T=st.integers(1, 300), E=st.sampled_from([1, 2, 4, 8, 16]), k=st.integers(1, 4),
+       BM=st.sampled_from([32, 64, 128, 256]), n4=st.integers(1, 90), ksteps=st.integers(1, 5),
+       epi=st.sampled_from(["plain", "weight", "silu"]), packed=st.booleans(),
+       dt=st.sampled_from([torch.bfloat16, torch.float16]), seed=st.integers(0, 10 ** 6))
+def test_gpu_grouped_gemm_any_shape(ops, dev, T, E, k, BM, n4, ksteps, epi, packed, dt, seed):
+    from oracle import torch_formulations
+    from sarathi_amd.layers import pack_expert_weights
+    k = min(k, E)
+    K = 64 * ksteps
+    N = 4 * n4 * (2 if epi == "silu" else 1)
+    if packed and epi == "silu" and (N // 2) % 32:
+        N = 64 * ((N // 2 + 31) // 32)        # packed gate / up tiles must not straddle
+    g = gen(seed)
+    gating = torch.randn((T, E), generator=g, dtype=torch.float32)
+    w = torch.empty((T, k))
+    ids = torch.empty((T, k), dtype=torch.int32)
+    src = torch.empty((T, k), dtype=torch.int32)
+    c_oracle.topk_softmax(w, ids, src, gating)
+    s, e, p = _align_oracle(ids, E, BM)
+    A = randn((T, K), g, dt, std=0.5)
+    B = randn((E, N, K), g, dt, std=0.5)
+    full = torch.zeros((T, k, N), dtype=dt)
+    torch_formulations.moe_grouped_gemm(A, B, full, w, s, e, p, T * k, BM, k, epi == "weight")
+    if epi == "silu":
+        want = torch.empty((T * k, N // 2), dtype=dt)
+        torch_formulations.silu_and_mul(want, full.view(-1, N))
+    else:
+        want = full.view(T * k, N)
+    got = torch.full(want.shape, 5.0, dtype=dt, device=dev)
+    Bd = B.to(dev)
+    ops.moe_ops.moe_grouped_gemm(A.to(dev), pack_expert_weights(Bd).data if packed else Bd, got,
+                                 w.to(dev), s.to(dev), e.to(dev), p.to(dev), T * k, BM, k,
+                                 epi == "weight", packed, N, epi == "silu")
+    got, want = got.float().cpu(), want.float()
+    tol = 2e-2 * want.abs().max().item() + 2e-2 * want.abs()
+    assert bool(((got - want).abs() <= tol).all()), "max diff %.4g" % (got - want).abs().max().item()
