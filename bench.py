@@ -332,6 +332,56 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    # ---- the other configurations of the same path (reported beside the headline workload) ----
+    # C1: the fused norm at the 512-token shape that is also the CPU-sized case; C5: the four ops at
+    # Llama-3-70B widths, T = 4608 (4096-token chunk + 512 decodes), one GPU, unsharded.
+    def measure_shape(Tn, Hn, nq, nkv, dff, which):
+        rows = {}
+        wn = dev_randn((Hn,))
+        table = cache_dev
+        posn = hybrid_positions(Tn, Tn - Tn // 9, gen(4), prefill_start=4096,
+                                max_pos=8192).to(dev) if "rotary_embedding" in which else None
+
+        def sized_ring(nbytes, make):
+            return [make() for _ in range(max(2, int(COLD_FOOTPRINT // nbytes) + 1))]
+        plan = {
+            "fused_add_rms_norm": (4 * Tn * Hn * BF16 + Hn * BF16,
+                                   lambda: (dev_randn((Tn, Hn)), dev_randn((Tn, Hn))),
+                                   lambda a: LN.fused_add_rms_norm(a[0], a[1], wn, 1e-5)),
+            "rms_norm": (2 * Tn * Hn * BF16 + Hn * BF16,
+                         lambda: (dev_randn((Tn, Hn)), dev_randn((Tn, Hn))),
+                         lambda a: LN.rms_norm(a[1], a[0], wn, 1e-5)),
+            "rotary_embedding": (2 * Tn * (nq + nkv) * D * BF16 + Tn * 8 + Tn * D * BF16,
+                                 lambda: dev_randn((Tn, (nq + 2 * nkv) * D)),
+                                 lambda a: ROPE.rotary_embedding(
+                                     posn, *a.split([nq * D, nkv * D, nkv * D], dim=-1)[:2], D,
+                                     table, True)),
+            "silu_and_mul": (3 * Tn * dff * BF16,
+                             lambda: (dev_randn((Tn, 2 * dff)),
+                                      torch.empty((Tn, dff), dtype=torch.bfloat16, device=dev)),
+                             lambda a: ACT.silu_and_mul(a[1], a[0])),
+        }
+        for name in which:
+            nbytes, make, fn = plan[name]
+            r = sized_ring(nbytes, make)
+            us = time_op(fn, r, max(20, args.steps // 2))
+            gbs = nbytes / us * 1e-3
+            rows[name] = {"bytes": nbytes, "cold": {"us": round(us, 3), "GBps": round(gbs, 1),
+                                                   "frac_of_peak": round(gbs / HBM_PEAK_GBS, 4)},
+                          "ring_sets": len(r)}
+            del r
+            torch.cuda.empty_cache()
+        return rows
+
+    other_configs = {
+        "fused_add_rms_norm [512, 4096] (CPU-sized case)":
+            measure_shape(512, 4096, 32, 8, 14336, ["fused_add_rms_norm"]),
+        "Llama-3-70B widths, T=4608: norm [4608, 8192], rope q[4608, 8192] k[4608, 1024], "
+        "silu_and_mul [4608, 57344]":
+            measure_shape(4608, 8192, 64, 8, 28672,
+                          ["fused_add_rms_norm", "rms_norm", "rotary_embedding", "silu_and_mul"]),
+    }
+
     silu_us = per_op["silu_and_mul"]["cold"]["us"]
     silu_gbs = BYTES["silu_and_mul"] / silu_us * 1e-3
     roofline = {
@@ -373,6 +423,34 @@ def main():
             times.append(time.perf_counter() - t_start)
         times.sort()
         med = times[len(times) // 2]
+
+        # a CPU column for every op of the table (median of a few repetitions, same formulations)
+        def cpu_us(fn, reps=5):
+            fn()
+            ts = []
+            for _ in range(reps):
+                t0 = time.perf_counter()
+                fn()
+                ts.append(time.perf_counter() - t0)
+            return round(sorted(ts)[len(ts) // 2] * 1e6, 1)
+        cnorm = torch.empty_like(cx)
+        cgating = gating.cpu()
+        ctw, cti, cts = tw.cpu(), ti.cpu(), ts.cpu()
+        csorted, cexp, cpost = sorted_ids.cpu(), expert_ids.cpu(), post_pad.cpu()
+        cpu_cols = {
+            "fused_add_rms_norm": lambda: cpu_ops.fused_add_rms_norm(cx, cr, cw, 1e-5),
+            "rms_norm": lambda: cpu_ops.rms_norm(cnorm, cx, cw, 1e-5),
+            "rotary_embedding": lambda: cpu_ops.rotary_embedding(cpos, cq, ck, D, cache_cpu, True),
+            "silu_and_mul": lambda: cpu_ops.silu_and_mul(cact, cgu),
+            "topk_softmax": lambda: cpu_ops.topk_softmax(ctw, cti, cts, cgating),
+            "moe_align_block_size": lambda: cpu_ops.moe_align_block_size(
+                cti, MOE_E, MOE_B, csorted, cexp, cpost),
+        }
+        for name, fn in cpu_cols.items():
+            per_op[name]["cpu_us"] = cpu_us(fn)
+        c1x, c1r = randn((512, H), cg), randn((512, H), cg)
+        other_configs["fused_add_rms_norm [512, 4096] (CPU-sized case)"]["fused_add_rms_norm"][
+            "cpu_us"] = cpu_us(lambda: cpu_ops.fused_add_rms_norm(c1x, c1r, cw, 1e-5), reps=20)
         cpu = {
             "value": round(step_bytes / med * 1e-9, 2), "unit": "GB/s",
             "cores": torch.get_num_threads(), "kind": "port",
@@ -403,6 +481,7 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "per_op": per_op,
+        "other_configs": other_configs,
         "plain_copy_same_bytes_cold": copy_ref,
     }
     print(json.dumps(out))
