@@ -71,14 +71,6 @@ template <int DT> SK_DEV f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
 // rows of both halves, whichever way the hardware groups the lanes of a 128-bit read.
 SK_DEV int lds_slot(int r, int c) { return (c + 2 * (r & 3) + ((r >> 2) & 1)) & 7; }
 
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
-// outstanding global load (its release fence drains vmcnt), i.e. for the weight and token
-// prefetches that are meant to stay in flight across the barrier; here a wave waits for its own
-// LDS operations and then meets the others.
-SK_DEV void lds_barrier() {
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
 struct MoeGemmArgs {
   const void* a;            // [tokens, K]
   const void* b;            // [E, N, K]

@@ -72,7 +72,7 @@ __global__ __launch_bounds__(64 * WAVES) void rms_norm_row_kernel(
   ss = wave64_sum(ss);
   if constexpr (WAVES > 1) {
     if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = ss;
-    __syncthreads();
+    lds_barrier();  // the residual stores and weight loads issued above stay in flight
     float t = partial[0];
 #pragma unroll
     for (int k = 1; k < WAVES; ++k) t += partial[k];

@@ -157,6 +157,17 @@ template <int DT> SK_DEV void store_elem(void* base, int64_t i, float v) {
   else reinterpret_cast<_Float16*>(base)[i] = (_Float16)v;
 }
 
+// ---- workgroup barrier for LDS exchanges ---------------------------------------
+
+// Orders LDS traffic only.  __syncthreads() also waits for every outstanding global access of
+// the wave (its release fence drains vmcnt, which on gfx9 counts loads and stores alike), i.e.
+// for prefetches and streaming stores that are meant to stay in flight across the barrier;
+// here a wave waits for its own LDS operations and then meets the others.  Use it only where
+// the data exchanged through the barrier lives in LDS.
+SK_DEV void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // ---- wave64 reductions -------------------------------------------------------
 
 // Adds `v` across the 64 lanes of a wave; every lane returns the total.
