@@ -49,12 +49,15 @@ def pack_expert_weights(w: torch.Tensor) -> PackedExpertWeights:
     return PackedExpertWeights(tiles, (E, N, K))
 
 
-# (token, k) slots up to which fused_moe routes with the one-launch kernel (it covers 16384).
-# Off by default: measured on MI355X at 4096 tokens x top-2 of 8 experts the single launch takes
-# 13.7 us against 12.8 us for the two kernels back to back (the sorting workgroup has to read the
-# ids through device-coherent loads, which costs what the saved launch gains); it only pays when
-# the host, not the GPU, is the bottleneck of the launch sequence.
-FUSED_ROUTING_MAX_SLOTS = 0
+# fused_moe routes with the one-launch kernel (top-k + slot sort) up to this many (token, k) slots
+# and experts.  Measured on MI355X, launches issued back to back from Python, E = 8, top-2:
+#   tokens     16     256    1024   2304   4096
+#   two ops    7.3    7.6    8.6    11.0   13.4  us
+#   one launch 5.9    5.8    7.9    11.0   14.1  us
+# Small batches gain a launch; from a few thousand slots on the sorting workgroup's device-coherent
+# reads of the ids cost more than the launch saved (and at 64 experts x top-6 there is no gain).
+FUSED_ROUTING_MAX_SLOTS = 2048
+FUSED_ROUTING_MAX_EXPERTS = 16
 # silu_and_mul inside the gate/up GEMM's epilogue (same bits as the separate kernel)
 FUSE_SILU_AND_MUL = True
 CHUNK_SIZE = 64 * 1024     # tokens per pass, as in the reference (fused_moe.py:437)
@@ -223,7 +226,7 @@ def fused_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
         assert num_expert_group is not None and topk_group is not None
         topk_weights, topk_ids = grouped_topk(hidden_states, gating_output, topk, renormalize,
                                               num_expert_group, topk_group)
-    elif 0 < num_tokens * topk <= FUSED_ROUTING_MAX_SLOTS:
+    elif 0 < num_tokens * topk <= FUSED_ROUTING_MAX_SLOTS and E <= FUSED_ROUTING_MAX_EXPERTS:
         # small batches are launch-latency bound: routing and slot sort in one launch
         config = try_get_optimal_moe_config(tuple(w1.shape), tuple(w2.shape), topk, num_tokens,
                                             override_config=override_config,

@@ -124,19 +124,21 @@ def test_fused_moe_forward(ops, dev, T, E, k, H, I, renorm):
 
 
 def test_fused_moe_with_one_launch_routing(ops, dev, monkeypatch):
-    """fused_moe with the routing + slot sort done by the single fused launch: same bits."""
-    from sarathi_amd import layers
+    """fused_moe with the routing + slot sort done by the single fused launch (the default for small
+    batches) and by the two separate kernels: same bits."""
     import importlib
     fm = importlib.import_module("sarathi_amd.layers.fused_moe")   # the module, not the function
+    from sarathi_amd import layers
     T, E, k, H, I = 300, 8, 2, 256, 512
     g = gen(21)
     x = randn((T, H), g, std=1.0).to(dev)
     w1 = randn((E, 2 * I, H), g, std=H ** -0.5).to(dev)
     w2 = randn((E, H, I), g, std=I ** -0.5).to(dev)
     gating = torch.randn((T, E), generator=g, dtype=torch.float32).to(dev)
-    want = layers.fused_moe(x, w1, w2, gating, k, True)
-    monkeypatch.setattr(fm, "FUSED_ROUTING_MAX_SLOTS", 16384)
-    got = layers.fused_moe(x, w1, w2, gating, k, True)
+    assert T * k <= fm.FUSED_ROUTING_MAX_SLOTS and E <= fm.FUSED_ROUTING_MAX_EXPERTS
+    got = layers.fused_moe(x, w1, w2, gating, k, True)                 # one-launch routing
+    monkeypatch.setattr(fm, "FUSED_ROUTING_MAX_SLOTS", 0)
+    want = layers.fused_moe(x, w1, w2, gating, k, True)                # two kernels
     assert torch.equal(got, want)
 
 
