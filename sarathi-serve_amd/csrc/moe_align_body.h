@@ -84,22 +84,25 @@ SK_DEV void align_single_workgroup(const IdT* __restrict__ ids, int64_t numel, i
     }
   };
   // cnt is indexed [e * W + wave]; only this wave touches its column, so plain LDS adds suffice
-  auto count_batch = [&](int64_t t0, const int (&e)[kAlignBatch]) {
+  // the matches of a batch are kept (`mt`) so that a resident chunk need not be matched again
+  // in the scatter pass
+  auto count_batch = [&](int64_t t0, const int (&e)[kAlignBatch], TileMatch (&mt)[kAlignBatch]) {
 #pragma unroll
     for (int u = 0; u < kAlignBatch; ++u) {
       if (t0 + u < tile_hi) {  // wave-uniform
         const bool valid = e[u] >= 0;
-        const TileMatch m = match_expert(e[u], valid, nbits);
-        if (valid && m.rank == 0) atomicAdd(&cnt[e[u] * W + wave], m.count);
+        mt[u] = match_expert(e[u], valid, nbits);
+        if (valid && mt[u].rank == 0) atomicAdd(&cnt[e[u] * W + wave], mt[u].count);
       }
     }
   };
-  auto scatter_batch = [&](int64_t t0, const int (&e)[kAlignBatch]) {
+  auto scatter_batch = [&](int64_t t0, const int (&e)[kAlignBatch],
+                           const TileMatch (&mt)[kAlignBatch], bool have_matches) {
 #pragma unroll
     for (int u = 0; u < kAlignBatch; ++u) {
       if (t0 + u < tile_hi) {
         const bool valid = e[u] >= 0;
-        const TileMatch m = match_expert(e[u], valid, nbits);
+        const TileMatch m = have_matches ? mt[u] : match_expert(e[u], valid, nbits);
         if (valid) {
           int32_t* c = &cnt[e[u] * W + wave];
           const int base = *c;  // every lane of the group reads before the leader's add below
@@ -113,14 +116,16 @@ SK_DEV void align_single_workgroup(const IdT* __restrict__ ids, int64_t numel, i
 
   // ---- 1. count
   int held[kAlignBatch];
+  TileMatch held_match[kAlignBatch];
   if (resident) {
     load_batch(tile_lo, held);
-    count_batch(tile_lo, held);
+    count_batch(tile_lo, held, held_match);
   } else {
     for (int64_t t0 = tile_lo; t0 < tile_hi; t0 += kAlignBatch) {
       int e[kAlignBatch];
+      TileMatch scratch[kAlignBatch];
       load_batch(t0, e);
-      count_batch(t0, e);
+      count_batch(t0, e, scratch);
     }
   }
   __syncthreads();
@@ -162,12 +167,12 @@ SK_DEV void align_single_workgroup(const IdT* __restrict__ ids, int64_t numel, i
 
   // ---- 3. scatter
   if (resident) {
-    scatter_batch(tile_lo, held);
+    scatter_batch(tile_lo, held, held_match, true);
   } else {
     for (int64_t t0 = tile_lo; t0 < tile_hi; t0 += kAlignBatch) {
       int e[kAlignBatch];
       load_batch(t0, e);
-      scatter_batch(t0, e);
+      scatter_batch(t0, e, held_match, false);
     }
   }
 
