@@ -260,7 +260,8 @@ int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c, const float*
  * slot_mapping[i] = page * page_size + entry.  The page table of a batch is the same for every
  * layer, so the append entry points accept the vector in place of the four index arrays
  * (slot_mapping != NULL: batch_indices, positions, kv_indices and kv_indptr are ignored and may be
- * NULL) and then need one index load per token instead of three dependent ones.
+ * NULL) and then need one index load per token instead of three dependent ones.  The mapping is
+ * int32: num_pages * page_size must stay below 2^31.
  */
 int sarathi_get_kv_slot_mapping(const int32_t* batch_indices, const int32_t* positions,
                                 const int32_t* kv_indices, const int32_t* kv_indptr,
