@@ -15,8 +15,12 @@ from oracle import c_oracle, paged_kv
 
 # SARATHI_TEST_EXAMPLES scales the number of drawn cases for an occasional longer soak
 _SCALE = max(1, int(os.environ.get("SARATHI_TEST_EXAMPLES", "1")))
-CPU = settings(max_examples=60 * _SCALE, deadline=None, suppress_health_check=list(HealthCheck))
-GPU = settings(max_examples=40 * _SCALE, deadline=None, suppress_health_check=list(HealthCheck))
+# the default run draws the same cases every time (a fixed regression set); a soak draws fresh ones
+_FIXED = "SARATHI_TEST_EXAMPLES" not in os.environ
+CPU = settings(max_examples=60 * _SCALE, deadline=None, derandomize=_FIXED, database=None,
+               suppress_health_check=list(HealthCheck))
+GPU = settings(max_examples=40 * _SCALE, deadline=None, derandomize=_FIXED, database=None,
+               suppress_health_check=list(HealthCheck))
 
 
 def _align_oracle(ids, E, B):
