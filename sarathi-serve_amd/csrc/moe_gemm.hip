@@ -27,10 +27,10 @@
 //                one 32x16 operand is contiguous in lane order, one fully
 //                coalesced load (~1.3-1.9x faster).  Weights are static, so
 //                packing them once at load time is free.
-//   tokens   shared by the four waves: gathered once per K-step into LDS
-//            (BM x 64 elements, 16-byte chunks rotated by row so that the
-//            operand reads are bank-conflict free), double buffered, one
-//            barrier per K-step.
+//   tokens   shared by the four waves: gathered once per K-step into LDS by
+//            buffer loads that write LDS directly (BM x 64 elements, 16-byte
+//            chunks rotated by row so that the operand reads are bank-conflict
+//            free), double buffered, one barrier per K-step.
 // Epilogues: plain; times the slot's routing weight (the down projection); or gated SiLU (the
 // gate/up projection followed by silu_and_mul, fused_moe.py:499-520): B then holds the gate rows
 // [0, N/2) and the up rows [N/2, N), a wave takes 32 gate rows and the 32 matching up rows as
@@ -70,6 +70,16 @@ template <int DT> SK_DEV f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
 // positions distinct both over eight consecutive rows of one half and over four consecutive
 // rows of both halves, whichever way the hardware groups the lanes of a 128-bit read.
 SK_DEV int lds_slot(int r, int c) { return (c + 2 * (r & 3) + ((r >> 2) & 1)) & 7; }
+
+// 16 bytes per lane from a buffer straight into LDS: lane l lands at lds_base + 16 l
+// (lds_base is uniform over the wave).  Completion is tracked by the wave's vmcnt.
+SK_DEV void dma_load16_to_lds(rsrc_t r, u32x4* lds_base, uint32_t byte_off) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(
+      r, (__attribute__((address_space(3))) void*)lds_base, 16, byte_off, 0, 0, 0);
+}
+
+// Waits until at most N vector-memory operations of this wave are outstanding.
+template <int N> SK_DEV void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
 struct MoeGemmArgs {
   const void* a;            // [tokens, K]
@@ -157,9 +167,10 @@ void moe_gemm_kernel(MoeGemmArgs g) {
                   : buf_load16<kCached>(rb, w_off[nt] + (uint32_t)(k0 + s * 16) * 2u);
   };
 
-  // ---- tokens: each thread gathers chunk `tid & 7` of rows (tid >> 3) + ROWS_PER_PASS j.
+  // ---- tokens: per K-step each thread moves one 16-byte chunk of rows (tid >> 3) +
+  // ROWS_PER_PASS j from global memory straight into LDS (no register staging).
   // A is one buffer resource; padding slots get an offset at its end (every K offset added
-  // later keeps them beyond it without wrapping), so their loads return zeros without a branch.
+  // later keeps them beyond it without wrapping), so their loads deposit zeros without a branch.
   const rsrc_t ra = make_rsrc(g.a, g.a_bytes);
   const int a_chunk = tid & 7;
   uint32_t a_off[A_LOADS];
@@ -169,18 +180,18 @@ void moe_gemm_kernel(MoeGemmArgs g) {
     const int slot_index = pid_m * BM + r;
     const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
     a_off[j] = sid < g.num_valid
-                   ? (uint32_t)(sid / g.top_k) * (uint32_t)(g.a_row_stride * 2) + a_chunk * 16u
+                   ? (uint32_t)(sid / g.top_k) * (uint32_t)(g.a_row_stride * 2) +
+                         (uint32_t)((a_chunk - 2 * (r & 3) - ((r >> 2) & 1)) & 7) * 16u
                    : g.a_bytes;
   }
-  auto gather = [&](int k0, u32x4 (&regs)[A_LOADS]) {
-#pragma unroll
-    for (int j = 0; j < A_LOADS; ++j) regs[j] = buf_load16<kCached>(ra, a_off[j] + (uint32_t)k0 * 2u);
-  };
-  auto stage = [&](int buf, const u32x4 (&regs)[A_LOADS]) {
+  // LDS DMA: lane l of a wave deposits its 16 bytes at (wave-uniform base) + 16 l, i.e. at
+  // position l & 7 of row base_row + l / 8; the lane therefore fetches the chunk that the rotated
+  // layout keeps at that position (the inverse of lds_slot, folded into a_off above).
+  auto gather_to_lds = [&](int k0, int buf) {
 #pragma unroll
     for (int j = 0; j < A_LOADS; ++j) {
-      const int r = (tid >> 3) + ROWS_PER_PASS * j;
-      tok_lds[buf][r * 8 + lds_slot(r, a_chunk)] = regs[j];
+      const int base_row = (tid >> 6) * 8 + ROWS_PER_PASS * j;
+      dma_load16_to_lds(ra, &tok_lds[buf][base_row * 8], a_off[j] + (uint32_t)k0 * 2u);
     }
   };
   f32x16 acc[NT][MT];
@@ -197,13 +208,12 @@ void moe_gemm_kernel(MoeGemmArgs g) {
   // instead of for one step.
   const int steps = g.K / kGemmBK;
   int kstep = 0;
-  u32x4 w[NT][SUB], anext[A_LOADS];
-  gather(kstep * kGemmBK, anext);
+  u32x4 w[NT][SUB];
+  gather_to_lds(kstep * kGemmBK, 0);
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
     for (int s = 0; s < SUB; ++s) w[nt][s] = load_weight(nt, kstep * kGemmBK, s);
-  stage(0, anext);
   __syncthreads();
 
   // (Meeting the other waves one sub-step earlier, so that the next K-step's first operand read
@@ -223,7 +233,7 @@ void moe_gemm_kernel(MoeGemmArgs g) {
     const int cur = step & 1;
     kstep = kstep + 1 < steps ? kstep + 1 : 0;
     const int k_next = kstep * kGemmBK;
-    gather(k_next, anext);
+    gather_to_lds(k_next, cur ^ 1);
     u32x4 tokv[2][MT];
     read_tokens(cur, 0, tokv[0]);
     __builtin_amdgcn_sched_barrier(0);
@@ -242,7 +252,8 @@ void moe_gemm_kernel(MoeGemmArgs g) {
       // of the next sub-step ahead of its MFMAs
       __builtin_amdgcn_sched_barrier(0);
     }
-    stage(cur ^ 1, anext);
+    // the DMA of this step is older than the NT * SUB weight loads issued since
+    wait_vmcnt<NT * SUB>();
     lds_barrier();
   }
 
