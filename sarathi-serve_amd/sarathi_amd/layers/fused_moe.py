@@ -36,16 +36,30 @@ class PackedExpertWeights:
         return True
 
 
-def pack_expert_weights(w: torch.Tensor) -> PackedExpertWeights:
+def pack_expert_weights(w: torch.Tensor, inplace: bool = False) -> PackedExpertWeights:
     """[E, N, K] -> tiles of 32 rows x 16 columns stored as 64 lanes x 8 elements, lane =
     (n mod 32) + 32 * ((k mod 16) // 8).  K must be a multiple of 16; N is padded with zero rows
-    to a multiple of 32.  Do this once when the weights are loaded."""
+    to a multiple of 32.  Do this once when the weights are loaded.
+
+    ``inplace=True`` re-tiles expert by expert inside ``w``'s own storage (one expert's matrix of
+    temporary memory instead of a second copy of all weights); ``w`` then no longer holds the
+    row-major values and must only be used through the returned object.  Needs N % 32 == 0 and a
+    contiguous ``w``."""
     E, N, K = w.shape
     assert K % 16 == 0, "K must be a multiple of 16"
     n_pad = (N + 31) // 32 * 32
+
+    def tile(m: torch.Tensor) -> torch.Tensor:      # [n_pad, K] -> [n_pad/32, K/16, 2, 32, 8]
+        return m.reshape(n_pad // 32, 32, K // 16, 2, 8).permute(0, 2, 3, 1, 4).contiguous()
+
+    if inplace:
+        assert n_pad == N and w.is_contiguous(), "in-place packing needs N % 32 == 0, contiguous w"
+        for e in range(E):
+            w[e].view(-1).copy_(tile(w[e]).view(-1))
+        return PackedExpertWeights(w.view(E, N // 32, K // 16, 2, 32, 8), (E, N, K))
     if n_pad != N:
         w = torch.cat((w, w.new_zeros((E, n_pad - N, K))), dim=1)
-    tiles = w.reshape(E, n_pad // 32, 32, K // 16, 2, 8).permute(0, 1, 3, 4, 2, 5).contiguous()
+    tiles = torch.stack([tile(w[e]) for e in range(E)])
     return PackedExpertWeights(tiles, (E, N, K))
 
 

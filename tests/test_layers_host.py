@@ -112,3 +112,23 @@ def test_rmsnorm_module_state(L):
     n = L.RMSNorm(128, eps=1e-5, norm_name="input_layernorm", layer_id=10)
     assert n.weight.shape == (128,) and bool((n.weight == 1).all())
     assert n.variance_epsilon == 1e-5 and n.norm_name == "input_layernorm" and n.layer_id == 10
+
+
+def test_pack_expert_weights_layout_and_inplace():
+    """Element (e, n, k) lands in tile n // 32, block k // 16, half (k % 16) // 8, lane row n % 32,
+    element k % 8; the in-place variant produces the same bytes inside the original storage."""
+    import importlib
+    fm = importlib.import_module("sarathi_amd.layers.fused_moe")
+    E, N, K = 3, 64, 48
+    w = torch.arange(E * N * K, dtype=torch.float32).reshape(E, N, K)
+    packed = fm.pack_expert_weights(w)
+    assert packed.shape == (E, N, K) and packed.data.shape == (E, N // 32, K // 16, 2, 32, 8)
+    for e, n, k in [(0, 0, 0), (1, 33, 17), (2, 63, 47), (1, 5, 9), (0, 32, 8)]:
+        assert packed.data[e, n // 32, k // 16, (k % 16) // 8, n % 32, k % 8] == w[e, n, k]
+    w2 = w.clone()
+    ptr = w2.data_ptr()
+    packed2 = fm.pack_expert_weights(w2, inplace=True)
+    assert packed2.data.data_ptr() == ptr and torch.equal(packed2.data, packed.data)
+    # rows beyond N are zero padding
+    odd = fm.pack_expert_weights(torch.ones((1, 40, 16)))
+    assert odd.data.shape == (1, 2, 1, 2, 32, 8) and odd.data[0, 1, 0, :, 8:, :].abs().sum() == 0
