@@ -40,78 +40,19 @@
 // Workgroup ids are mapped so that the eight XCDs (id mod 8) each take their
 // own column blocks and walk the slot blocks fastest: workgroups that run
 // together on an XCD share the expert's weight tile in that XCD's L2.
-#include "vec16.h"
+#include "moe_gemm_common.h"
 #include "launch.h"
 
 namespace sarathi_hip {
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-
-constexpr int kGemmBN = 256;   // output columns per workgroup
-constexpr int kGemmBK = 64;    // K elements per pipeline step
-constexpr int kGemmWaveN = 64; // output columns per wave
-
-enum : int { kEpiPlain = 0, kEpiMulWeight = 1, kEpiGatedSilu = 2 };
-
-template <int DT> SK_DEV f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
-  if constexpr (DT == kBF16)
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-  else
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
-                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-}
-
-// Position (0..7) of 16-byte chunk c inside row r of the token tile in LDS.  Rows are 128 bytes,
-// i.e. exactly one pass over the 32 banks, so the bank group of an access is this position.
-// An operand read has lane (row r, half g) fetch chunk 2s + g; the rotation below makes the
-// positions distinct both over eight consecutive rows of one half and over four consecutive
-// rows of both halves, whichever way the hardware groups the lanes of a 128-bit read.
-SK_DEV int lds_slot(int r, int c) { return (c + 2 * (r & 3) + ((r >> 2) & 1)) & 7; }
-
-// 16 bytes per lane from a buffer straight into LDS: lane l lands at lds_base + 16 l
-// (lds_base is uniform over the wave).  Completion is tracked by the wave's vmcnt.
-SK_DEV void dma_load16_to_lds(rsrc_t r, u32x4* lds_base, uint32_t byte_off) {
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(
-      r, (__attribute__((address_space(3))) void*)lds_base, 16, byte_off, 0, 0, 0);
-}
-
-// Waits until at most N vector-memory operations of this wave are outstanding.
-template <int N> SK_DEV void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
-
-struct MoeGemmArgs {
-  const void* a;            // [tokens, K]
-  const void* b;            // [E, N, K]
-  void* c;                  // [tokens * top_k, N]
-  const float* topk_weights;        // flat [tokens * top_k] or null
-  const int32_t* sorted_token_ids;  // [em]
-  const int32_t* expert_ids;        // [ceil(em / BM)]
-  const int32_t* num_tokens_post_padded;
-  uint32_t a_bytes;         // extent of A in bytes; a_bytes + 2*K stays below 4 GiB
-  int64_t a_row_stride;     // elements
-  int64_t b_expert_stride;  // elements
-  int64_t c_row_stride;     // elements
-  int32_t num_valid;        // tokens * top_k
-  int32_t em;               // length of sorted_token_ids
-  int32_t N, K;
-  int32_t top_k;
-  int32_t m_blocks, n_blocks;
-};
-
-// A workgroup is four waves side by side, each owning all BM slots x 64 output columns.  At
-// BM = 256 a wave holds a 256 x 64 accumulator tile (256 registers, one wave per SIMD), which
-// halves the weight bytes loaded per flop: the fastest shape for row-major weights, whose loads
-// are the bottleneck (880 against 725 TFLOP/s at BM = 128); with packed weights BM = 128 at two
-// waves per SIMD wins (1060 against 910).  Eight-wave workgroups with two wave rows sharing each
-// weight tile through the L1 were measured slower than both.
-// Up to BM = 128, at least two waves per SIMD: with 128 accumulator registers per lane that
-// caps the other registers at 128, which the main loop meets anyway (106); without the bound
-// the epilogues that do arithmetic on the accumulators are allocated ~138 and the whole kernel
-// drops to one wave per SIMD (measured: 15 % slower).
+// A workgroup is four waves side by side, each owning all BM slots x 64 output columns, for
+// BM = 32, 64 and 128 (256-slot blocks run the kernel of moe_gemm_lds.hip).
+// At least two waves per SIMD: with 128 accumulator registers per lane (BM = 128) that caps the
+// other registers at 128, which the main loop meets anyway; without the bound the epilogues
+// that do arithmetic on the accumulators are allocated ~138 and the whole kernel drops to one
+// wave per SIMD (measured: 15 % slower).
 template <int DT, int BM, int EPI, bool PACKED>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM > 128 ? 1 : 2)))
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 void moe_gemm_kernel(MoeGemmArgs g) {
   constexpr bool MUL_WEIGHT = EPI == kEpiMulWeight;
   constexpr bool GATED = EPI == kEpiGatedSilu;
@@ -328,6 +269,10 @@ static int launch_moe_gemm(const MoeGemmArgs& g, int epilogue, bool packed, hipS
   return launch_status();
 }
 
+// moe_gemm_lds.hip: the 256-slot-block kernel with both operands shared through LDS
+int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int epilogue, bool packed, int dtype,
+                        hipStream_t st);
+
 }  // namespace sarathi_hip
 
 extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
@@ -392,12 +337,12 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
                      : (int32_t)((n + kGemmBN - 1) / kGemmBN);
   hipStream_t st = (hipStream_t)stream;
   const int mw = epilogue;
+  if (block_m == 256) return launch_moe_gemm_lds(g, c_cols, mw, packed, dtype, st);
 #define SK_GEMM(DT)                                                       \
   switch (block_m) {                                                      \
     case 32: return launch_moe_gemm<DT, 32>(g, mw, packed, st);           \
     case 64: return launch_moe_gemm<DT, 64>(g, mw, packed, st);           \
-    case 128: return launch_moe_gemm<DT, 128>(g, mw, packed, st);         \
-    default: return launch_moe_gemm<DT, 256>(g, mw, packed, st);          \
+    default: return launch_moe_gemm<DT, 128>(g, mw, packed, st);          \
   }
   if (dtype == kBF16) { SK_GEMM(kBF16) } else { SK_GEMM(kF16) }
 #undef SK_GEMM

@@ -1,0 +1,288 @@
+// Grouped expert GEMM, 256-slot blocks, both operands through LDS.
+//
+// Same computation and argument block as moe_gemm.hip.  That kernel feeds the weights from global
+// memory straight into registers, wave by wave; its counters show the vector-memory front end
+// (address / command FIFOs full for about as many cycles as the compute units are busy) as the
+// limit, i.e. the bytes every compute unit pulls through its L1 per flop.  Here a workgroup of
+// EIGHT waves owns 256 slots x 256 output columns: two wave rows of 128 slots share each weight
+// tile, and four wave columns share each token tile, both through LDS, so a compute unit loads
+// 64 KB per 64-deep K-step for 8.4 MFLOP instead of 96 KB.  Every wave still holds a 128 x 64
+// accumulator tile (128 registers), so two waves fit on a SIMD.
+//
+// Data movement: every global -> LDS transfer is a buffer load that writes LDS directly (no
+// register staging), issued one K-step ahead into the other half of a double buffer; one barrier
+// per K-step.
+//   tokens   256 rows x 128 bytes per K-step, 16-byte chunks rotated by row (bank-conflict-free
+//            operand reads), exactly as in moe_gemm.hip.
+//   weights  packed layout: the 32 operand blocks of 1 KiB a K-step needs (4 strips x 2 tiles x 4
+//            sub-steps) are copied as they are, lane order, and read back linearly.
+//            row-major layout: a strip's 64 rows x 128 bytes are fetched as whole 128-byte row
+//            segments (eight lanes per row: fully coalesced, unlike the per-lane 16-byte row
+//            reads of the register path) into the same rotated row layout as the tokens.
+//            Either way 32 KiB per K-step.
+// LDS: 2 x (32 KiB tokens + 32 KiB weights) = 128 KiB, requested as dynamic shared memory.
+#include "moe_gemm_common.h"
+#include "launch.h"
+
+namespace sarathi_hip {
+
+constexpr int kLdsBM = 256;                       // slots per workgroup
+constexpr int kLdsWaves = 8;                      // 2 wave rows x 4 wave columns
+constexpr int kLdsUnits = kLdsBM * 8;             // 16-byte units per operand buffer (32 KiB)
+constexpr int kLdsBytes = 4 * kLdsUnits * 16;     // tokens + weights, double buffered
+
+template <int DT, int EPI, bool PACKED>
+__global__ __launch_bounds__(64 * kLdsWaves) __attribute__((amdgpu_waves_per_eu(2)))
+void moe_gemm_lds_kernel(MoeGemmArgs g) {
+  constexpr bool MUL_WEIGHT = EPI == kEpiMulWeight;
+  constexpr bool GATED = EPI == kEpiGatedSilu;
+  constexpr int BM = kLdsBM, BN = 256;
+  constexpr int MT = 4, NT = 2, SUB = kGemmBK / 16;
+  extern __shared__ u32x4 lds[];
+  u32x4* const tok = lds;                 // [2][BM rows][8 units]
+  u32x4* const wgt = lds + 2 * kLdsUnits; // [2][2048 units]
+
+  // ---- which tile (same id -> tile map as the register kernel)
+  const unsigned id = blockIdx.x;
+  const unsigned xcd = id & 7u, t = id >> 3;
+  const int pid_m = t % g.m_blocks;
+  const int pid_n = (t / g.m_blocks) * 8 + xcd;
+  if (pid_n >= g.n_blocks) return;
+  if (pid_m * BM >= *g.num_tokens_post_padded) return;
+  const int expert = g.expert_ids[pid_m];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wn = wave & 3;          // wave column: weight strip of 64 rows
+  const int row0 = (wave >> 2) * 128;  // wave row: first slot of this wave inside the block
+  const int l32 = lane & 31, grp = lane >> 5;
+  const int half_n = g.N >> 1;      // gated: weight rows [half_n, N) are the up projection
+  const int n_tiles = (g.N + 31) >> 5;
+
+  // first weight row of strip `strip`, tile `nt` of this workgroup (gated: tile 0 holds 32 gate
+  // rows, tile 1 the matching up rows), or -1 when the strip lies beyond the matrix
+  auto tile_row0 = [&](int strip, int nt) {
+    if constexpr (GATED) {
+      const int gate0 = pid_n * (BN / 2) + strip * 32;
+      return gate0 < half_n ? gate0 + nt * half_n : -1;
+    } else {
+      const int n0 = pid_n * BN + strip * 64 + nt * 32;
+      return n0 < g.N ? n0 : -1;
+    }
+  };
+
+  // ---- weights: four DMA instructions per wave and K-step
+  const int64_t b_bytes = PACKED ? (int64_t)n_tiles * 32 * g.K * 2 : (int64_t)g.N * g.K * 2;
+  const rsrc_t rb = make_rsrc(
+      reinterpret_cast<const char*>(g.b) + (int64_t)expert * g.b_expert_stride * 2, (uint32_t)b_bytes);
+  uint32_t w_off[4];  // global byte offset at k = 0 of the piece this lane moves
+  int w_unit[4];      // LDS unit (wave-uniform) at which the instruction's 64 lanes start
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int q = wave * 4 + i;  // 0..31
+    if constexpr (PACKED) {
+      // block q = (strip * 2 + nt) * 4 + s: the 1 KiB operand block of sub-step s
+      const int strip = q >> 3, nt = (q >> 2) & 1, s = q & 3;
+      const int r0 = tile_row0(strip, nt);
+      w_off[i] = r0 >= 0 ? (uint32_t)(r0 >> 5) * (uint32_t)g.K * 64u + (uint32_t)s * 1024u + lane * 16u
+                         : 0x80000000u;
+      w_unit[i] = q * 64;
+    } else {
+      // instruction q covers rows [8 (q & 7), +8) of strip q >> 3; lane = (row, position)
+      const int strip = q >> 3, rr = (q & 7) * 8 + (lane >> 3);  // row inside the strip, 0..63
+      const int r0 = tile_row0(strip, rr >> 5);
+      const int n = r0 + (rr & 31);
+      const bool in_range = r0 >= 0 && (GATED ? (r0 - (rr >> 5) * half_n) + (rr & 31) < half_n
+                                              : n < g.N);
+      const int R = strip * 64 + rr;  // row inside the workgroup's weight tile
+      const int chunk = ((lane & 7) - 2 * (R & 3) - ((R >> 2) & 1)) & 7;
+      w_off[i] = in_range ? (uint32_t)n * (uint32_t)g.K * 2u + (uint32_t)chunk * 16u : 0x80000000u;
+      w_unit[i] = (strip * 64 + (q & 7) * 8) * 8;
+    }
+  }
+  auto dma_weights = [&](int k0, int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t koff = PACKED ? (uint32_t)(k0 >> 4) * 1024u : (uint32_t)k0 * 2u;
+      dma_load16_to_lds(rb, wgt + buf * kLdsUnits + w_unit[i], w_off[i] + koff);
+    }
+  };
+
+  // ---- tokens: four DMA instructions per wave and K-step (64 rows per pass)
+  const rsrc_t ra = make_rsrc(g.a, g.a_bytes);
+  uint32_t a_off[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int r = (tid >> 3) + 64 * j;
+    const int slot_index = pid_m * BM + r;
+    const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
+    const int chunk = ((tid & 7) - 2 * (r & 3) - ((r >> 2) & 1)) & 7;
+    a_off[j] = sid < g.num_valid
+                   ? (uint32_t)(sid / g.top_k) * (uint32_t)(g.a_row_stride * 2) + (uint32_t)chunk * 16u
+                   : g.a_bytes;
+  }
+  auto dma_tokens = [&](int k0, int buf) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      dma_load16_to_lds(ra, tok + buf * kLdsUnits + (wave * 8 + 64 * j) * 8,
+                        a_off[j] + (uint32_t)k0 * 2u);
+  };
+
+  // ---- operand reads of one 16-deep sub-step
+  auto read_operands = [&](int buf, int s, u32x4 (&tv)[MT], u32x4 (&wv)[NT]) {
+    const u32x4* tb = tok + buf * kLdsUnits;
+    const u32x4* wb = wgt + buf * kLdsUnits;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int r = row0 + mt * 32 + l32;
+      tv[mt] = tb[r * 8 + lds_slot(r, 2 * s + grp)];
+    }
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      if constexpr (PACKED) {
+        wv[nt] = wb[((wn * 2 + nt) * 4 + s) * 64 + lane];
+      } else {
+        const int R = wn * 64 + nt * 32 + l32;
+        wv[nt] = wb[R * 8 + lds_slot(R, 2 * s + grp)];
+      }
+    }
+  };
+
+  f32x16 acc[NT][MT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[nt][mt][i] = 0.f;
+
+  const int steps = g.K / kGemmBK;
+  int kstep = 0;
+  dma_tokens(0, 0);
+  dma_weights(0, 0);
+  wait_vmcnt<0>();
+  lds_barrier();
+
+  // Branch-free loop: the last step fetches the wrapped-around first K-step again (never used).
+  // A buffer is overwritten only after every wave has passed the barrier that followed its
+  // last reads of it.
+  for (int step = 0; step < steps; ++step) {
+    const int cur = step & 1;
+    kstep = kstep + 1 < steps ? kstep + 1 : 0;
+    dma_tokens(kstep * kGemmBK, cur ^ 1);
+    dma_weights(kstep * kGemmBK, cur ^ 1);
+    u32x4 tv[2][MT], wv[2][NT];
+    read_operands(cur, 0, tv[0], wv[0]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = 0; s < SUB; ++s) {
+      if (s + 1 < SUB) read_operands(cur, s + 1, tv[(s + 1) & 1], wv[(s + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);  // reads of s + 1 are in flight under the MFMAs of s
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[nt][mt] = mfma32<DT>(wv[s & 1][nt], tv[s & 1][mt], acc[nt][mt]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    wait_vmcnt<0>();  // this step's transfers (issued a whole K-step ago) have landed
+    lds_barrier();
+  }
+
+  // ---- epilogue: lane holds, per accumulator quad, 4 consecutive columns of one token
+  const int n_wave0 = GATED ? pid_n * (BN / 2) + wn * 32 : pid_n * BN + wn * 64;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int slot_index = pid_m * BM + row0 + mt * 32 + l32;
+    const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
+    if (sid >= g.num_valid) continue;
+    float scale = 1.f;
+    if constexpr (MUL_WEIGHT) scale = g.topk_weights[sid];
+    char* crow = reinterpret_cast<char*>(g.c) + (int64_t)sid * g.c_row_stride * 2;
+    if constexpr (GATED) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n_wave0 + q * 8 + grp * 4;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float x = rnd<DT>(acc[0][mt][q * 4 + e]), y = rnd<DT>(acc[1][mt][q * 4 + e]);
+          v[e] = rnd<DT>(silu_f32(x)) * y;
+        }
+        if (n + 3 < half_n) {
+          u32x2 out = {pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
+          *reinterpret_cast<u32x2*>(crow + (int64_t)n * 2) = out;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < half_n) store_elem<DT>(crow, n + e, v[e]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = n_wave0 + nt * 32 + q * 8 + grp * 4;
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            v[e] = acc[nt][mt][q * 4 + e];
+            if constexpr (MUL_WEIGHT) v[e] *= scale;
+          }
+          if (n + 3 < g.N) {
+            u32x2 out = {pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
+            *reinterpret_cast<u32x2*>(crow + (int64_t)n * 2) = out;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n + e < g.N) store_elem<DT>(crow, n + e, v[e]);
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int DT, int EPI, bool PACKED>
+static int launch_one(const MoeGemmArgs& g, dim3 grid, hipStream_t st) {
+  auto kernel = moe_gemm_lds_kernel<DT, EPI, PACKED>;
+  // more LDS than the default per-workgroup limit: opt in once per kernel and device
+  static bool raised[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return SARATHI_ERR_LAUNCH;
+  if (!raised[dev]) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess)
+      return SARATHI_ERR_LAUNCH;
+    raised[dev] = true;
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(64 * kLdsWaves), kLdsBytes, st, g);
+  return launch_status();
+}
+
+// Entry used by sarathi_moe_grouped_gemm for 256-slot blocks.  `g` is complete except for
+// n_blocks, which depends on the epilogue.
+int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int epilogue, bool packed, int dtype,
+                        hipStream_t st) {
+  const int64_t cols_per_block = epilogue == kEpiGatedSilu ? 128 : 256;
+  g.n_blocks = (int32_t)((out_cols + cols_per_block - 1) / cols_per_block);
+  const int64_t blocks = (int64_t)((g.n_blocks + 7) / 8) * g.m_blocks * 8;
+  if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)blocks);
+#define SK_PICK(DT)                                                                        \
+  switch (epilogue) {                                                                      \
+    case kEpiMulWeight:                                                                    \
+      return packed ? launch_one<DT, kEpiMulWeight, true>(g, grid, st)                     \
+                    : launch_one<DT, kEpiMulWeight, false>(g, grid, st);                   \
+    case kEpiGatedSilu:                                                                    \
+      return packed ? launch_one<DT, kEpiGatedSilu, true>(g, grid, st)                     \
+                    : launch_one<DT, kEpiGatedSilu, false>(g, grid, st);                   \
+    default:                                                                               \
+      return packed ? launch_one<DT, kEpiPlain, true>(g, grid, st)                         \
+                    : launch_one<DT, kEpiPlain, false>(g, grid, st);                       \
+  }
+  if (dtype == kBF16) { SK_PICK(kBF16) } else { SK_PICK(kF16) }
+#undef SK_PICK
+}
+
+}  // namespace sarathi_hip
