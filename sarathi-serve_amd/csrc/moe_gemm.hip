@@ -270,8 +270,8 @@ static int launch_moe_gemm(const MoeGemmArgs& g, int epilogue, bool packed, hipS
 }
 
 // moe_gemm_lds.hip: the 256-slot-block kernel with both operands shared through LDS
-int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int epilogue, bool packed, int dtype,
-                        hipStream_t st);
+int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, bool packed,
+                        int dtype, hipStream_t st);
 
 }  // namespace sarathi_hip
 
@@ -337,7 +337,9 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
                      : (int32_t)((n + kGemmBN - 1) / kGemmBN);
   hipStream_t st = (hipStream_t)stream;
   const int mw = epilogue;
-  if (block_m == 256) return launch_moe_gemm_lds(g, c_cols, mw, packed, dtype, st);
+  // 256-slot blocks always, and row-major weights from 64 slots on, go through LDS
+  if (block_m == 256 || (!packed && block_m >= 64))
+    return launch_moe_gemm_lds(g, c_cols, block_m, mw, packed, dtype, st);
 #define SK_GEMM(DT)                                                       \
   switch (block_m) {                                                      \
     case 32: return launch_moe_gemm<DT, 32>(g, mw, packed, st);           \

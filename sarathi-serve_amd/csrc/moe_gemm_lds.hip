@@ -1,10 +1,11 @@
-// Grouped expert GEMM, 256-slot blocks, both operands through LDS.
+// Grouped expert GEMM with both operands through LDS (256-slot blocks; row-major weights at any
+// block size from 64).
 //
 // Same computation and argument block as moe_gemm.hip.  That kernel feeds the weights from global
 // memory straight into registers, wave by wave; its counters show the vector-memory front end
 // (address / command FIFOs full for about as many cycles as the compute units are busy) as the
 // limit, i.e. the bytes every compute unit pulls through its L1 per flop.  Here a workgroup of
-// EIGHT waves owns 256 slots x 256 output columns: two wave rows of 128 slots share each weight
+// EIGHT waves owns BM (256) slots x 256 output columns: two wave rows of BM / 2 slots share each weight
 // tile, and four wave columns share each token tile, both through LDS, so a compute unit loads
 // 64 KB per 64-deep K-step for 8.4 MFLOP instead of 96 KB.  Every wave still holds a 128 x 64
 // accumulator tile (128 registers), so two waves fit on a SIMD.
@@ -20,27 +21,33 @@
 //            segments (eight lanes per row: fully coalesced, unlike the per-lane 16-byte row
 //            reads of the register path) into the same rotated row layout as the tokens.
 //            Either way 32 KiB per K-step.
-// LDS: 2 x (32 KiB tokens + 32 KiB weights) = 128 KiB, requested as dynamic shared memory.
+// LDS: 2 x (BM x 128 bytes of tokens + 32 KiB of weights), 128 KiB at BM = 256, requested as dynamic
+// shared memory.
 #include "moe_gemm_common.h"
 #include "launch.h"
 
 namespace sarathi_hip {
 
-constexpr int kLdsBM = 256;                       // slots per workgroup
-constexpr int kLdsWaves = 8;                      // 2 wave rows x 4 wave columns
-constexpr int kLdsUnits = kLdsBM * 8;             // 16-byte units per operand buffer (32 KiB)
-constexpr int kLdsBytes = 4 * kLdsUnits * 16;     // tokens + weights, double buffered
+constexpr int kLdsWaves = 8;          // 2 wave rows x 4 wave columns
+constexpr int kLdsWgtUnits = 256 * 8;  // 16-byte units of a weight buffer (256 rows x 128 bytes)
+// dynamic shared memory of a workgroup with BM slots: tokens + weights, double buffered
+constexpr int lds_bytes(int BM) { return 2 * (BM * 8 + kLdsWgtUnits) * 16; }
 
-template <int DT, int EPI, bool PACKED>
+// BM = 256 (two waves per SIMD, 128 KiB of LDS: one workgroup per compute unit) is the large-batch
+// shape; BM = 64 and 128 exist for row-major weights at small batches, where the coalesced
+// row-segment fetch is what matters and several workgroups share a compute unit.
+template <int DT, int BM, int EPI, bool PACKED>
 __global__ __launch_bounds__(64 * kLdsWaves) __attribute__((amdgpu_waves_per_eu(2)))
 void moe_gemm_lds_kernel(MoeGemmArgs g) {
   constexpr bool MUL_WEIGHT = EPI == kEpiMulWeight;
   constexpr bool GATED = EPI == kEpiGatedSilu;
-  constexpr int BM = kLdsBM, BN = 256;
-  constexpr int MT = 4, NT = 2, SUB = kGemmBK / 16;
+  constexpr int BN = 256;
+  constexpr int MT = BM / 64, NT = 2, SUB = kGemmBK / 16;  // a wave row holds BM / 2 slots
+  constexpr int TOK_UNITS = BM * 8;
+  constexpr int TOK_PASSES = BM / 64;  // 512 threads move 64 rows of 128 bytes per pass
   extern __shared__ u32x4 lds[];
-  u32x4* const tok = lds;                 // [2][BM rows][8 units]
-  u32x4* const wgt = lds + 2 * kLdsUnits; // [2][2048 units]
+  u32x4* const tok = lds;                  // [2][BM rows][8 units]
+  u32x4* const wgt = lds + 2 * TOK_UNITS;  // [2][256 rows][8 units]
 
   // ---- which tile (same id -> tile map as the register kernel)
   const unsigned id = blockIdx.x;
@@ -53,7 +60,7 @@ void moe_gemm_lds_kernel(MoeGemmArgs g) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wn = wave & 3;          // wave column: weight strip of 64 rows
-  const int row0 = (wave >> 2) * 128;  // wave row: first slot of this wave inside the block
+  const int row0 = (wave >> 2) * (BM / 2);  // wave row: first slot of this wave inside the block
   const int l32 = lane & 31, grp = lane >> 5;
   const int half_n = g.N >> 1;      // gated: weight rows [half_n, N) are the up projection
   const int n_tiles = (g.N + 31) >> 5;
@@ -103,15 +110,15 @@ void moe_gemm_lds_kernel(MoeGemmArgs g) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint32_t koff = PACKED ? (uint32_t)(k0 >> 4) * 1024u : (uint32_t)k0 * 2u;
-      dma_load16_to_lds(rb, wgt + buf * kLdsUnits + w_unit[i], w_off[i] + koff);
+      dma_load16_to_lds(rb, wgt + buf * kLdsWgtUnits + w_unit[i], w_off[i] + koff);
     }
   };
 
-  // ---- tokens: four DMA instructions per wave and K-step (64 rows per pass)
+  // ---- tokens: one DMA instruction per wave, pass and K-step (64 rows per pass)
   const rsrc_t ra = make_rsrc(g.a, g.a_bytes);
-  uint32_t a_off[4];
+  uint32_t a_off[TOK_PASSES];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < TOK_PASSES; ++j) {
     const int r = (tid >> 3) + 64 * j;
     const int slot_index = pid_m * BM + r;
     const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
@@ -122,15 +129,15 @@ void moe_gemm_lds_kernel(MoeGemmArgs g) {
   }
   auto dma_tokens = [&](int k0, int buf) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      dma_load16_to_lds(ra, tok + buf * kLdsUnits + (wave * 8 + 64 * j) * 8,
+    for (int j = 0; j < TOK_PASSES; ++j)
+      dma_load16_to_lds(ra, tok + buf * TOK_UNITS + (wave * 8 + 64 * j) * 8,
                         a_off[j] + (uint32_t)k0 * 2u);
   };
 
   // ---- operand reads of one 16-deep sub-step
   auto read_operands = [&](int buf, int s, u32x4 (&tv)[MT], u32x4 (&wv)[NT]) {
-    const u32x4* tb = tok + buf * kLdsUnits;
-    const u32x4* wb = wgt + buf * kLdsUnits;
+    const u32x4* tb = tok + buf * TOK_UNITS;
+    const u32x4* wb = wgt + buf * kLdsWgtUnits;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const int r = row0 + mt * 32 + l32;
@@ -243,43 +250,54 @@ void moe_gemm_lds_kernel(MoeGemmArgs g) {
   }
 }
 
-template <int DT, int EPI, bool PACKED>
+template <int DT, int BM, int EPI, bool PACKED>
 static int launch_one(const MoeGemmArgs& g, dim3 grid, hipStream_t st) {
-  auto kernel = moe_gemm_lds_kernel<DT, EPI, PACKED>;
+  auto kernel = moe_gemm_lds_kernel<DT, BM, EPI, PACKED>;
+  constexpr int bytes = lds_bytes(BM);
   // more LDS than the default per-workgroup limit: opt in once per kernel and device
   static bool raised[64] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return SARATHI_ERR_LAUNCH;
   if (!raised[dev]) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess)
+                            hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
       return SARATHI_ERR_LAUNCH;
     raised[dev] = true;
   }
-  hipLaunchKernelGGL(kernel, grid, dim3(64 * kLdsWaves), kLdsBytes, st, g);
+  hipLaunchKernelGGL(kernel, grid, dim3(64 * kLdsWaves), bytes, st, g);
   return launch_status();
 }
 
-// Entry used by sarathi_moe_grouped_gemm for 256-slot blocks.  `g` is complete except for
-// n_blocks, which depends on the epilogue.
-int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int epilogue, bool packed, int dtype,
-                        hipStream_t st) {
+template <int DT, int BM>
+static int launch_epilogue(const MoeGemmArgs& g, dim3 grid, int epilogue, bool packed,
+                           hipStream_t st) {
+  switch (epilogue) {
+    case kEpiMulWeight:
+      return packed ? launch_one<DT, BM, kEpiMulWeight, true>(g, grid, st)
+                    : launch_one<DT, BM, kEpiMulWeight, false>(g, grid, st);
+    case kEpiGatedSilu:
+      return packed ? launch_one<DT, BM, kEpiGatedSilu, true>(g, grid, st)
+                    : launch_one<DT, BM, kEpiGatedSilu, false>(g, grid, st);
+    default:
+      return packed ? launch_one<DT, BM, kEpiPlain, true>(g, grid, st)
+                    : launch_one<DT, BM, kEpiPlain, false>(g, grid, st);
+  }
+}
+
+// Entry used by sarathi_moe_grouped_gemm; block_m is 64, 128 or 256.  `g` is complete except
+// for n_blocks, which depends on the epilogue.
+int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, bool packed,
+                        int dtype, hipStream_t st) {
   const int64_t cols_per_block = epilogue == kEpiGatedSilu ? 128 : 256;
   g.n_blocks = (int32_t)((out_cols + cols_per_block - 1) / cols_per_block);
   const int64_t blocks = (int64_t)((g.n_blocks + 7) / 8) * g.m_blocks * 8;
   if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)blocks);
-#define SK_PICK(DT)                                                                        \
-  switch (epilogue) {                                                                      \
-    case kEpiMulWeight:                                                                    \
-      return packed ? launch_one<DT, kEpiMulWeight, true>(g, grid, st)                     \
-                    : launch_one<DT, kEpiMulWeight, false>(g, grid, st);                   \
-    case kEpiGatedSilu:                                                                    \
-      return packed ? launch_one<DT, kEpiGatedSilu, true>(g, grid, st)                     \
-                    : launch_one<DT, kEpiGatedSilu, false>(g, grid, st);                   \
-    default:                                                                               \
-      return packed ? launch_one<DT, kEpiPlain, true>(g, grid, st)                         \
-                    : launch_one<DT, kEpiPlain, false>(g, grid, st);                       \
+#define SK_PICK(DT)                                                                      \
+  switch (block_m) {                                                                     \
+    case 64: return launch_epilogue<DT, 64>(g, grid, epilogue, packed, st);              \
+    case 128: return launch_epilogue<DT, 128>(g, grid, epilogue, packed, st);            \
+    default: return launch_epilogue<DT, 256>(g, grid, epilogue, packed, st);             \
   }
   if (dtype == kBF16) { SK_PICK(kBF16) } else { SK_PICK(kF16) }
 #undef SK_PICK
