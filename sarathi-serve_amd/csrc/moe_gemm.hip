@@ -25,7 +25,7 @@
 //                unit, not the MFMA pipe, the limit (~22-36 % of peak);
 //              packed    [E, N/32, K/16, 64 lanes, 8]: the 1 KiB a wave needs for
 //                one 32x16 operand is contiguous in lane order, one fully
-//                coalesced load (~1.3-1.9x faster).  Weights are static, so
+//                coalesced load (~1.3-1.9x faster in this kernel).  Weights are static, so
 //                packing them once at load time is free.
 //   tokens   shared by the four waves: gathered once per K-step into LDS by
 //            buffer loads that write LDS directly (BM x 64 elements, 16-byte
