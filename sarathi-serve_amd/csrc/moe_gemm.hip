@@ -65,11 +65,8 @@ void moe_gemm_kernel(MoeGemmArgs g) {
   __shared__ u32x4 tok_lds[2][BM * 8];  // [buffer][row * 8 + rotated chunk]
 
   // ---- which tile
-  const unsigned id = blockIdx.x;
-  const unsigned xcd = id & 7u, t = id >> 3;
-  const int pid_m = t % g.m_blocks;
-  const int pid_n = (t / g.m_blocks) * 8 + xcd;
-  if (pid_n >= g.n_blocks) return;
+  int pid_m, pid_n;
+  if (!tile_of_block(g, blockIdx.x, pid_m, pid_n)) return;
   if (pid_m * BM >= *g.num_tokens_post_padded) return;
   const int expert = g.expert_ids[pid_m];
 
@@ -122,7 +119,7 @@ void moe_gemm_kernel(MoeGemmArgs g) {
     const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
     a_off[j] = sid < g.num_valid
                    ? (uint32_t)(sid / g.top_k) * (uint32_t)(g.a_row_stride * 2) +
-                         (uint32_t)((a_chunk - 2 * (r & 3) - ((r >> 2) & 1)) & 7) * 16u
+                         (uint32_t)lds_chunk_at(r, a_chunk) * 16u
                    : g.a_bytes;
   }
   // LDS DMA: lane l of a wave deposits its 16 bytes at (wave-uniform base) + 16 l, i.e. at
@@ -163,40 +160,59 @@ void moe_gemm_kernel(MoeGemmArgs g) {
   // interleaved: the last step simply loads the wrapped-around "next" K-step again (issued,
   // never used), and the token operands of sub-step s + 1 are read from LDS before the MFMAs
   // of sub-step s are issued.
-  auto read_tokens = [&](int buf, int s, u32x4 (&tokv)[MT]) {
+  // Padding sits at the end of an expert's run of slots, so the last block of every expert has
+  // 32-slot tiles without a single valid slot (half a block per expert on average).  mt_live is
+  // one past the last tile of this block that holds a valid slot; the loop is compiled once per
+  // possible value, each copy branch-free and without the LDS reads and MFMAs of the tiles
+  // beyond it.
+  int mt_live = 0;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int r = mt * 32 + l32;
-      tokv[mt] = tok_lds[buf][r * 8 + lds_slot(r, 2 * s + grp)];
+  for (int mt = 0; mt < MT; ++mt) {
+    const int slot_index = pid_m * BM + mt * 32 + l32;
+    const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
+    if (__ballot(sid < g.num_valid) != 0ull) mt_live = mt + 1;
+  }
+  auto k_loop = [&](auto live_tag) {
+    constexpr int LIVE = decltype(live_tag)::value;  // tiles 0 .. LIVE - 1 are computed
+    auto read_live_tokens = [&](int buf, int s, u32x4 (&tokv)[MT]) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        if (mt >= LIVE) continue;
+        const int r = mt * 32 + l32;
+        tokv[mt] = tok_lds[buf][r * 8 + lds_slot(r, 2 * s + grp)];
+      }
+    };
+    for (int step = 0; step < steps; ++step) {
+      const int cur = step & 1;
+      kstep = kstep + 1 < steps ? kstep + 1 : 0;
+      const int k_next = kstep * kGemmBK;
+      gather_to_lds(k_next, cur ^ 1);
+      u32x4 tokv[2][MT];
+      read_live_tokens(cur, 0, tokv[0]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < SUB; ++s) {
+        if (s + 1 < SUB) read_live_tokens(cur, s + 1, tokv[(s + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);  // LDS reads of s + 1 are in flight under the MFMAs of s
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            if (mt >= LIVE) continue;
+            acc[nt][mt] = mfma32<DT>(w[nt][s], tokv[s & 1][mt], acc[nt][mt]);
+          }
+          w[nt][s] = load_weight(nt, k_next, s);  // the slot is free again: refill it
+        }
+        // keep this sub-step's loads here (a full K-step ahead of their use) and the LDS reads
+        // of the next sub-step ahead of its MFMAs
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // the DMA of this step is older than the NT * SUB weight loads issued since
+      wait_vmcnt<NT * SUB>();
+      lds_barrier();
     }
   };
-  for (int step = 0; step < steps; ++step) {
-    const int cur = step & 1;
-    kstep = kstep + 1 < steps ? kstep + 1 : 0;
-    const int k_next = kstep * kGemmBK;
-    gather_to_lds(k_next, cur ^ 1);
-    u32x4 tokv[2][MT];
-    read_tokens(cur, 0, tokv[0]);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int s = 0; s < SUB; ++s) {
-      if (s + 1 < SUB) read_tokens(cur, s + 1, tokv[(s + 1) & 1]);
-      __builtin_amdgcn_sched_barrier(0);  // LDS reads of s + 1 are in flight under the MFMAs of s
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-          acc[nt][mt] = mfma32<DT>(w[nt][s], tokv[s & 1][mt], acc[nt][mt]);
-        w[nt][s] = load_weight(nt, k_next, s);  // the slot is free again: refill it
-      }
-      // keep this sub-step's loads here (a full K-step ahead of their use) and the LDS reads
-      // of the next sub-step ahead of its MFMAs
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    // the DMA of this step is older than the NT * SUB weight loads issued since
-    wait_vmcnt<NT * SUB>();
-    lds_barrier();
-  }
+  call_with_live<MT>(mt_live, k_loop);
 
   // ---- epilogue: lane holds, per accumulator quad, 4 consecutive columns of one token
 #pragma unroll
@@ -335,6 +351,7 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
   g.m_blocks = (int32_t)((sorted_len + block_m - 1) / block_m);
   g.n_blocks = gated ? (int32_t)((c_cols + kGemmBN / 2 - 1) / (kGemmBN / 2))
                      : (int32_t)((n + kGemmBN - 1) / kGemmBN);
+  g.group_n = kGemmGroupN;
   hipStream_t st = (hipStream_t)stream;
   const int mw = epilogue;
   // 256-slot blocks always, and row-major weights from 64 slots on, go through LDS

@@ -50,11 +50,8 @@ void moe_gemm_lds_kernel(MoeGemmArgs g) {
   u32x4* const wgt = lds + 2 * TOK_UNITS;  // [2][256 rows][8 units]
 
   // ---- which tile (same id -> tile map as the register kernel)
-  const unsigned id = blockIdx.x;
-  const unsigned xcd = id & 7u, t = id >> 3;
-  const int pid_m = t % g.m_blocks;
-  const int pid_n = (t / g.m_blocks) * 8 + xcd;
-  if (pid_n >= g.n_blocks) return;
+  int pid_m, pid_n;
+  if (!tile_of_block(g, blockIdx.x, pid_m, pid_n)) return;
   if (pid_m * BM >= *g.num_tokens_post_padded) return;
   const int expert = g.expert_ids[pid_m];
 
@@ -101,7 +98,7 @@ void moe_gemm_lds_kernel(MoeGemmArgs g) {
       const bool in_range = r0 >= 0 && (GATED ? (r0 - (rr >> 5) * half_n) + (rr & 31) < half_n
                                               : n < g.N);
       const int R = strip * 64 + rr;  // row inside the workgroup's weight tile
-      const int chunk = ((lane & 7) - 2 * (R & 3) - ((R >> 2) & 1)) & 7;
+      const int chunk = lds_chunk_at(R, lane & 7);
       w_off[i] = in_range ? (uint32_t)n * (uint32_t)g.K * 2u + (uint32_t)chunk * 16u : 0x80000000u;
       w_unit[i] = (strip * 64 + (q & 7) * 8) * 8;
     }
@@ -122,7 +119,7 @@ void moe_gemm_lds_kernel(MoeGemmArgs g) {
     const int r = (tid >> 3) + 64 * j;
     const int slot_index = pid_m * BM + r;
     const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
-    const int chunk = ((tid & 7) - 2 * (r & 3) - ((r >> 2) & 1)) & 7;
+    const int chunk = lds_chunk_at(r, tid & 7);
     a_off[j] = sid < g.num_valid
                    ? (uint32_t)(sid / g.top_k) * (uint32_t)(g.a_row_stride * 2) + (uint32_t)chunk * 16u
                    : g.a_bytes;
@@ -134,26 +131,6 @@ void moe_gemm_lds_kernel(MoeGemmArgs g) {
                         a_off[j] + (uint32_t)k0 * 2u);
   };
 
-  // ---- operand reads of one 16-deep sub-step
-  auto read_operands = [&](int buf, int s, u32x4 (&tv)[MT], u32x4 (&wv)[NT]) {
-    const u32x4* tb = tok + buf * TOK_UNITS;
-    const u32x4* wb = wgt + buf * kLdsWgtUnits;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int r = row0 + mt * 32 + l32;
-      tv[mt] = tb[r * 8 + lds_slot(r, 2 * s + grp)];
-    }
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      if constexpr (PACKED) {
-        wv[nt] = wb[((wn * 2 + nt) * 4 + s) * 64 + lane];
-      } else {
-        const int R = wn * 64 + nt * 32 + l32;
-        wv[nt] = wb[R * 8 + lds_slot(R, 2 * s + grp)];
-      }
-    }
-  };
-
   f32x16 acc[NT][MT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
@@ -163,37 +140,84 @@ void moe_gemm_lds_kernel(MoeGemmArgs g) {
       for (int i = 0; i < 16; ++i) acc[nt][mt][i] = 0.f;
 
   const int steps = g.K / kGemmBK;
-  int kstep = 0;
+  auto wrap = [&](int k) { return k < steps ? k : k - steps; };  // k < 2 * steps
   dma_tokens(0, 0);
   dma_weights(0, 0);
   wait_vmcnt<0>();
   lds_barrier();
-
-  // Branch-free loop: the last step fetches the wrapped-around first K-step again (never used).
-  // A buffer is overwritten only after every wave has passed the barrier that followed its
-  // last reads of it.
-  for (int step = 0; step < steps; ++step) {
-    const int cur = step & 1;
-    kstep = kstep + 1 < steps ? kstep + 1 : 0;
-    dma_tokens(kstep * kGemmBK, cur ^ 1);
-    dma_weights(kstep * kGemmBK, cur ^ 1);
-    u32x4 tv[2][MT], wv[2][NT];
-    read_operands(cur, 0, tv[0], wv[0]);
-    __builtin_amdgcn_sched_barrier(0);
+  int kstep = wrap(1);  // the K-step whose transfers are in flight
+  dma_tokens(kstep * kGemmBK, 1);
+  dma_weights(kstep * kGemmBK, 1);
+  // Padding sits at the end of an expert's run of slots, so the last block of every expert has
+  // 32-slot tiles without a single valid slot.  mt_live is one past the last tile of this wave's
+  // rows that holds a valid slot; the loop is compiled once per possible value, each copy
+  // branch-free and without the token reads and MFMAs of the tiles beyond it (a wave without any
+  // live tile only moves data and meets the others at the barriers).
+  int mt_live = 0;
 #pragma unroll
-    for (int s = 0; s < SUB; ++s) {
-      if (s + 1 < SUB) read_operands(cur, s + 1, tv[(s + 1) & 1], wv[(s + 1) & 1]);
-      __builtin_amdgcn_sched_barrier(0);  // reads of s + 1 are in flight under the MFMAs of s
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-          acc[nt][mt] = mfma32<DT>(wv[s & 1][nt], tv[s & 1][mt], acc[nt][mt]);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    wait_vmcnt<0>();  // this step's transfers (issued a whole K-step ago) have landed
-    lds_barrier();
+  for (int mt = 0; mt < MT; ++mt) {
+    const int slot_index = pid_m * BM + row0 + mt * 32 + l32;
+    const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
+    if (__ballot(sid < g.num_valid) != 0ull) mt_live = mt + 1;
   }
+
+  // Branch-free loop: the last two steps fetch wrapped-around K-steps again (never used).
+  // The barrier of a step sits before its LAST sub-step, whose operands are already in registers:
+  // once every wave is past it, the other buffer has landed and nobody reads this one any more,
+  // so the transfers two K-steps ahead start into this buffer and the first operands of the next
+  // step are read while the matrix cores still work on this step's last sub-step.
+  auto k_loop = [&](auto live_tag) {
+    constexpr int LIVE = decltype(live_tag)::value;  // tiles 0 .. LIVE - 1 are computed
+    auto read_operands = [&](int buf, int s, u32x4 (&tv)[MT], u32x4 (&wv)[NT]) {
+      const u32x4* tb = tok + buf * TOK_UNITS;
+      const u32x4* wb = wgt + buf * kLdsWgtUnits;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        if (mt >= LIVE) continue;
+        const int r = row0 + mt * 32 + l32;
+        tv[mt] = tb[r * 8 + lds_slot(r, 2 * s + grp)];
+      }
+      if (LIVE == 0) return;
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        if constexpr (PACKED) {
+          wv[nt] = wb[((wn * 2 + nt) * 4 + s) * 64 + lane];
+        } else {
+          const int R = wn * 64 + nt * 32 + l32;
+          wv[nt] = wb[R * 8 + lds_slot(R, 2 * s + grp)];
+        }
+      }
+    };
+    u32x4 tv[2][MT], wv[2][NT];
+    read_operands(0, 0, tv[0], wv[0]);
+    for (int step = 0; step < steps; ++step) {
+      const int cur = step & 1;
+#pragma unroll
+      for (int s = 0; s < SUB; ++s) {
+        if (s + 1 < SUB) {
+          read_operands(cur, s + 1, tv[(s + 1) & 1], wv[(s + 1) & 1]);
+        } else {
+          wait_vmcnt<0>();  // the next step's transfers (issued a whole K-step ago) have landed
+          lds_barrier();
+          kstep = wrap(kstep + 1);
+          dma_tokens(kstep * kGemmBK, cur);
+          dma_weights(kstep * kGemmBK, cur);
+          read_operands(cur ^ 1, 0, tv[0], wv[0]);
+        }
+        __builtin_amdgcn_sched_barrier(0);  // the reads are in flight under the MFMAs of s
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            if (mt >= LIVE) continue;
+            acc[nt][mt] = mfma32<DT>(wv[s & 1][nt], tv[s & 1][mt], acc[nt][mt]);
+          }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  call_with_live<MT>(mt_live, k_loop);
+  wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup ends
 
   // ---- epilogue: lane holds, per accumulator quad, 4 consecutive columns of one token
   const int n_wave0 = GATED ? pid_n * (BN / 2) + wn * 32 : pid_n * BN + wn * 64;

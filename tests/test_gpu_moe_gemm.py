@@ -69,6 +69,43 @@ def test_grouped_gemm_matches_formulation(ops, dev, dtype, T, E, k, BM, N, K, mu
     assert torch.equal(got2, got)
 
 
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("BM", [64, 128, 256])
+def test_grouped_gemm_padding_anywhere_in_a_block(ops, dev, BM, packed):
+    """The kernels skip 32-slot tiles that hold no valid slot.  moe_align_block_size puts padding
+    at the end of a block, but the operator accepts any slot order: shuffle the slots inside every
+    block so that valid slots sit behind, between and in front of all-padding tiles; also covers
+    blocks whose first or second half is entirely padding.  Same products per output, so the
+    result must equal the unshuffled run bit for bit and the formulation within tolerance."""
+    T, E, k, N, K = 90, 8, 2, 320, 192
+    _, w, ids, s, e, p = _route(T, E, k, BM, 31 + BM)
+    g = gen(BM)
+    A = randn((T, K), g, std=0.5)
+    Bw = randn((E, N, K), g, std=0.5)
+    want = torch.zeros((T, k, N), dtype=torch.bfloat16)
+    torch_formulations.moe_grouped_gemm(A, Bw, want, w, s, e, p, T * k, BM, k, True)
+    used = int(p.item())
+    shuffled = s.clone()
+    for b in range(used // BM):
+        perm = torch.randperm(BM, generator=g)
+        shuffled[b * BM:(b + 1) * BM] = s[b * BM:(b + 1) * BM][perm]
+    # one block with its valid slots moved to the very end (every earlier tile all padding)
+    blk = s[:BM]
+    shuffled[:BM] = torch.cat([blk[blk >= T * k], blk[blk < T * k]])
+    Bd = Bw.to(dev)
+    if packed:
+        from sarathi_amd.layers import pack_expert_weights
+        Bd = pack_expert_weights(Bd).data
+    outs = []
+    for order in (s, shuffled):
+        got = torch.full((T, k, N), 7.0, dtype=torch.bfloat16, device=dev)
+        ops.moe_ops.moe_grouped_gemm(A.to(dev), Bd, got, w.to(dev), order.to(dev), e.to(dev),
+                                     p.to(dev), T * k, BM, k, True, packed, N)
+        outs.append(got)
+    _close(outs[0], want, "aligned order")
+    assert torch.equal(outs[0], outs[1])
+
+
 def test_grouped_gemm_second_stage_addressing(ops, dev):
     """top_k = 1 addressing of the down projection: A rows are slots (tokens * topk of them)."""
     T, E, k, BM, N, K = 200, 8, 2, 64, 256, 128
