@@ -46,18 +46,21 @@
 namespace sarathi_hip {
 
 // A workgroup is four waves side by side, each owning all BM slots x 64 output columns, for
-// BM = 32, 64 and 128 (256-slot blocks run the kernel of moe_gemm_lds.hip).
+// BM = 32, 64 and 128.  BM = 256 (packed weights only) is eight waves, two rows of four: each row
+// owns 128 slots, the token tile in LDS serves all eight, and the second row's weight loads hit
+// in the compute unit's L1 behind the first row's.
 // At least two waves per SIMD: with 128 accumulator registers per lane (BM = 128) that caps the
 // other registers at 128, which the main loop meets anyway; without the bound the epilogues
 // that do arithmetic on the accumulators are allocated ~138 and the whole kernel drops to one
 // wave per SIMD (measured: 15 % slower).
 template <int DT, int BM, int EPI, bool PACKED>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+__global__ __launch_bounds__(BM == 256 ? 512 : 256) __attribute__((amdgpu_waves_per_eu(2)))
 void moe_gemm_kernel(MoeGemmArgs g) {
   constexpr bool MUL_WEIGHT = EPI == kEpiMulWeight;
   constexpr bool GATED = EPI == kEpiGatedSilu;
-  constexpr int THREADS = 256;
-  constexpr int MT = BM / 32;          // token tiles per wave
+  constexpr int WR = BM == 256 ? 2 : 1;  // wave rows
+  constexpr int THREADS = 256 * WR;
+  constexpr int MT = BM / WR / 32;     // token tiles per wave
   constexpr int NT = kGemmWaveN / 32;  // weight tiles per wave
   constexpr int SUB = kGemmBK / 16;    // MFMA sub-steps per K-step
   constexpr int ROWS_PER_PASS = THREADS / 8;
@@ -71,7 +74,8 @@ void moe_gemm_kernel(MoeGemmArgs g) {
   const int expert = g.expert_ids[pid_m];
 
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = tid >> 6;  // output columns [64 wave, 64 wave + 64)
+  const int wave = (tid >> 6) & 3;  // wave column: output columns [64 wave, 64 wave + 64)
+  const int row0 = (tid >> 8) * (BM / WR);  // wave row: first slot of this wave inside the block
   const int l32 = lane & 31, grp = lane >> 5;
 
   // ---- weights: buffer resource over the expert's matrix; rows >= N read as zero
@@ -168,7 +172,7 @@ void moe_gemm_kernel(MoeGemmArgs g) {
   int mt_live = 0;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const int slot_index = pid_m * BM + mt * 32 + l32;
+    const int slot_index = pid_m * BM + row0 + mt * 32 + l32;
     const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
     if (__ballot(sid < g.num_valid) != 0ull) mt_live = mt + 1;
   }
@@ -178,7 +182,7 @@ void moe_gemm_kernel(MoeGemmArgs g) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         if (mt >= LIVE) continue;
-        const int r = mt * 32 + l32;
+        const int r = row0 + mt * 32 + l32;
         tokv[mt] = tok_lds[buf][r * 8 + lds_slot(r, 2 * s + grp)];
       }
     };
@@ -217,7 +221,7 @@ void moe_gemm_kernel(MoeGemmArgs g) {
   // ---- epilogue: lane holds, per accumulator quad, 4 consecutive columns of one token
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const int slot_index = pid_m * BM + mt * 32 + l32;
+    const int slot_index = pid_m * BM + row0 + mt * 32 + l32;
     const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
     if (sid >= g.num_valid) continue;
     float scale = 1.f;
@@ -271,9 +275,14 @@ static int launch_moe_gemm(const MoeGemmArgs& g, int epilogue, bool packed, hipS
   const int64_t groups = (g.n_blocks + 7) / 8;
   const int64_t blocks = groups * g.m_blocks * 8;
   if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
-  const dim3 grid((unsigned)blocks), block(256);
+  const dim3 grid((unsigned)blocks), block(BM == 256 ? 512 : 256);
 #define SK_LAUNCH(EP, PK) \
   hipLaunchKernelGGL((moe_gemm_kernel<DT, BM, EP, PK>), grid, block, 0, st, g)
+  if constexpr (BM == 256) {  // eight waves: packed weights only
+    if (epilogue == kEpiMulWeight) SK_LAUNCH(kEpiMulWeight, true);
+    else if (epilogue == kEpiGatedSilu) SK_LAUNCH(kEpiGatedSilu, true);
+    else SK_LAUNCH(kEpiPlain, true);
+  } else
   if (epilogue == kEpiMulWeight) {
     if (packed) SK_LAUNCH(kEpiMulWeight, true); else SK_LAUNCH(kEpiMulWeight, false);
   } else if (epilogue == kEpiGatedSilu) {
@@ -285,9 +294,9 @@ static int launch_moe_gemm(const MoeGemmArgs& g, int epilogue, bool packed, hipS
   return launch_status();
 }
 
-// moe_gemm_lds.hip: the 256-slot-block kernel with both operands shared through LDS
-int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, bool packed,
-                        int dtype, hipStream_t st);
+// moe_gemm_lds.hip: row-major weights, both operands shared through LDS
+int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, int dtype,
+                        hipStream_t st);
 
 }  // namespace sarathi_hip
 
@@ -354,13 +363,13 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
   g.group_n = kGemmGroupN;
   hipStream_t st = (hipStream_t)stream;
   const int mw = epilogue;
-  // 256-slot blocks always, and row-major weights from 64 slots on, go through LDS
-  if (block_m == 256 || (!packed && block_m >= 64))
-    return launch_moe_gemm_lds(g, c_cols, block_m, mw, packed, dtype, st);
+  // row-major weights go through LDS from 64-slot blocks on
+  if (!packed && block_m >= 64) return launch_moe_gemm_lds(g, c_cols, block_m, mw, dtype, st);
 #define SK_GEMM(DT)                                                       \
   switch (block_m) {                                                      \
     case 32: return launch_moe_gemm<DT, 32>(g, mw, packed, st);           \
     case 64: return launch_moe_gemm<DT, 64>(g, mw, packed, st);           \
+    case 256: return launch_moe_gemm<DT, 256>(g, mw, packed, st);         \
     default: return launch_moe_gemm<DT, 128>(g, mw, packed, st);          \
   }
   if (dtype == kBF16) { SK_GEMM(kBF16) } else { SK_GEMM(kF16) }

@@ -1,26 +1,23 @@
-// Grouped expert GEMM with both operands through LDS (256-slot blocks; row-major weights at any
-// block size from 64).
+// Grouped expert GEMM for row-major ([E, N, K]) expert weights, both operands through LDS, at
+// block sizes 64, 128 and 256.
 //
 // Same computation and argument block as moe_gemm.hip.  That kernel feeds the weights from global
-// memory straight into registers, wave by wave; its counters show the vector-memory front end
-// (address / command FIFOs full for about as many cycles as the compute units are busy) as the
-// limit, i.e. the bytes every compute unit pulls through its L1 per flop.  Here a workgroup of
-// EIGHT waves owns BM (256) slots x 256 output columns: two wave rows of BM / 2 slots share each weight
+// memory straight into registers, wave by wave: with the packed layout every such load is one
+// contiguous KiB, but with row-major weights a lane's 16 bytes come from 32 different rows, 8 KB
+// or more apart, and the vector-memory front end becomes the limit.  Here a workgroup of EIGHT
+// waves owns BM slots x 256 output columns: two wave rows of BM / 2 slots share each weight
 // tile, and four wave columns share each token tile, both through LDS, so a compute unit loads
-// 64 KB per 64-deep K-step for 8.4 MFLOP instead of 96 KB.  Every wave still holds a 128 x 64
-// accumulator tile (128 registers), so two waves fit on a SIMD.
+// 64 KB per 64-deep K-step for 8.4 MFLOP (BM = 256).  Every wave holds a (BM / 2) x 64
+// accumulator tile (128 registers at BM = 256), so two waves fit on a SIMD.
 //
 // Data movement: every global -> LDS transfer is a buffer load that writes LDS directly (no
 // register staging), issued one K-step ahead into the other half of a double buffer; one barrier
 // per K-step.
-//   tokens   256 rows x 128 bytes per K-step, 16-byte chunks rotated by row (bank-conflict-free
+//   tokens   BM rows x 128 bytes per K-step, 16-byte chunks rotated by row (bank-conflict-free
 //            operand reads), exactly as in moe_gemm.hip.
-//   weights  packed layout: the 32 operand blocks of 1 KiB a K-step needs (4 strips x 2 tiles x 4
-//            sub-steps) are copied as they are, lane order, and read back linearly.
-//            row-major layout: a strip's 64 rows x 128 bytes are fetched as whole 128-byte row
-//            segments (eight lanes per row: fully coalesced, unlike the per-lane 16-byte row
-//            reads of the register path) into the same rotated row layout as the tokens.
-//            Either way 32 KiB per K-step.
+//   weights  a strip's 64 rows x 128 bytes are fetched as whole 128-byte row segments (eight
+//            lanes per row: fully coalesced) into the same rotated row layout as the tokens;
+//            32 KiB per K-step.
 // LDS: 2 x (BM x 128 bytes of tokens + 32 KiB of weights), 128 KiB at BM = 256, requested as dynamic
 // shared memory.
 #include "moe_gemm_common.h"
@@ -36,7 +33,7 @@ constexpr int lds_bytes(int BM) { return 2 * (BM * 8 + kLdsWgtUnits) * 16; }
 // BM = 256 (two waves per SIMD, 128 KiB of LDS: one workgroup per compute unit) is the large-batch
 // shape; BM = 64 and 128 exist for row-major weights at small batches, where the coalesced
 // row-segment fetch is what matters and several workgroups share a compute unit.
-template <int DT, int BM, int EPI, bool PACKED>
+template <int DT, int BM, int EPI>
 __global__ __launch_bounds__(64 * kLdsWaves) __attribute__((amdgpu_waves_per_eu(2)))
 void moe_gemm_lds_kernel(MoeGemmArgs g) {
   constexpr bool MUL_WEIGHT = EPI == kEpiMulWeight;
@@ -60,7 +57,6 @@ void moe_gemm_lds_kernel(MoeGemmArgs g) {
   const int row0 = (wave >> 2) * (BM / 2);  // wave row: first slot of this wave inside the block
   const int l32 = lane & 31, grp = lane >> 5;
   const int half_n = g.N >> 1;      // gated: weight rows [half_n, N) are the up projection
-  const int n_tiles = (g.N + 31) >> 5;
 
   // first weight row of strip `strip`, tile `nt` of this workgroup (gated: tile 0 holds 32 gate
   // rows, tile 1 the matching up rows), or -1 when the strip lies beyond the matrix
@@ -75,7 +71,7 @@ void moe_gemm_lds_kernel(MoeGemmArgs g) {
   };
 
   // ---- weights: four DMA instructions per wave and K-step
-  const int64_t b_bytes = PACKED ? (int64_t)n_tiles * 32 * g.K * 2 : (int64_t)g.N * g.K * 2;
+  const int64_t b_bytes = (int64_t)g.N * g.K * 2;
   const rsrc_t rb = make_rsrc(
       reinterpret_cast<const char*>(g.b) + (int64_t)expert * g.b_expert_stride * 2, (uint32_t)b_bytes);
   uint32_t w_off[4];  // global byte offset at k = 0 of the piece this lane moves
@@ -83,32 +79,21 @@ void moe_gemm_lds_kernel(MoeGemmArgs g) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int q = wave * 4 + i;  // 0..31
-    if constexpr (PACKED) {
-      // block q = (strip * 2 + nt) * 4 + s: the 1 KiB operand block of sub-step s
-      const int strip = q >> 3, nt = (q >> 2) & 1, s = q & 3;
-      const int r0 = tile_row0(strip, nt);
-      w_off[i] = r0 >= 0 ? (uint32_t)(r0 >> 5) * (uint32_t)g.K * 64u + (uint32_t)s * 1024u + lane * 16u
-                         : 0x80000000u;
-      w_unit[i] = q * 64;
-    } else {
-      // instruction q covers rows [8 (q & 7), +8) of strip q >> 3; lane = (row, position)
-      const int strip = q >> 3, rr = (q & 7) * 8 + (lane >> 3);  // row inside the strip, 0..63
-      const int r0 = tile_row0(strip, rr >> 5);
-      const int n = r0 + (rr & 31);
-      const bool in_range = r0 >= 0 && (GATED ? (r0 - (rr >> 5) * half_n) + (rr & 31) < half_n
-                                              : n < g.N);
-      const int R = strip * 64 + rr;  // row inside the workgroup's weight tile
-      const int chunk = lds_chunk_at(R, lane & 7);
-      w_off[i] = in_range ? (uint32_t)n * (uint32_t)g.K * 2u + (uint32_t)chunk * 16u : 0x80000000u;
-      w_unit[i] = (strip * 64 + (q & 7) * 8) * 8;
-    }
+    // instruction q covers rows [8 (q & 7), +8) of strip q >> 3; lane = (row, position)
+    const int strip = q >> 3, rr = (q & 7) * 8 + (lane >> 3);  // row inside the strip, 0..63
+    const int r0 = tile_row0(strip, rr >> 5);
+    const int n = r0 + (rr & 31);
+    const bool in_range = r0 >= 0 && (GATED ? (r0 - (rr >> 5) * half_n) + (rr & 31) < half_n
+                                            : n < g.N);
+    const int R = strip * 64 + rr;  // row inside the workgroup's weight tile
+    const int chunk = lds_chunk_at(R, lane & 7);
+    w_off[i] = in_range ? (uint32_t)n * (uint32_t)g.K * 2u + (uint32_t)chunk * 16u : 0x80000000u;
+    w_unit[i] = (strip * 64 + (q & 7) * 8) * 8;
   }
   auto dma_weights = [&](int k0, int buf) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t koff = PACKED ? (uint32_t)(k0 >> 4) * 1024u : (uint32_t)k0 * 2u;
-      dma_load16_to_lds(rb, wgt + buf * kLdsWgtUnits + w_unit[i], w_off[i] + koff);
-    }
+    for (int i = 0; i < 4; ++i)
+      dma_load16_to_lds(rb, wgt + buf * kLdsWgtUnits + w_unit[i], w_off[i] + (uint32_t)k0 * 2u);
   };
 
   // ---- tokens: one DMA instruction per wave, pass and K-step (64 rows per pass)
@@ -180,12 +165,8 @@ void moe_gemm_lds_kernel(MoeGemmArgs g) {
       if (LIVE == 0) return;
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-        if constexpr (PACKED) {
-          wv[nt] = wb[((wn * 2 + nt) * 4 + s) * 64 + lane];
-        } else {
-          const int R = wn * 64 + nt * 32 + l32;
-          wv[nt] = wb[R * 8 + lds_slot(R, 2 * s + grp)];
-        }
+        const int R = wn * 64 + nt * 32 + l32;
+        wv[nt] = wb[R * 8 + lds_slot(R, 2 * s + grp)];
       }
     };
     u32x4 tv[2][MT], wv[2][NT];
@@ -274,9 +255,9 @@ void moe_gemm_lds_kernel(MoeGemmArgs g) {
   }
 }
 
-template <int DT, int BM, int EPI, bool PACKED>
+template <int DT, int BM, int EPI>
 static int launch_one(const MoeGemmArgs& g, dim3 grid, hipStream_t st) {
-  auto kernel = moe_gemm_lds_kernel<DT, BM, EPI, PACKED>;
+  auto kernel = moe_gemm_lds_kernel<DT, BM, EPI>;
   constexpr int bytes = lds_bytes(BM);
   // more LDS than the default per-workgroup limit: opt in once per kernel and device
   static bool raised[64] = {};
@@ -293,25 +274,18 @@ static int launch_one(const MoeGemmArgs& g, dim3 grid, hipStream_t st) {
 }
 
 template <int DT, int BM>
-static int launch_epilogue(const MoeGemmArgs& g, dim3 grid, int epilogue, bool packed,
-                           hipStream_t st) {
+static int launch_epilogue(const MoeGemmArgs& g, dim3 grid, int epilogue, hipStream_t st) {
   switch (epilogue) {
-    case kEpiMulWeight:
-      return packed ? launch_one<DT, BM, kEpiMulWeight, true>(g, grid, st)
-                    : launch_one<DT, BM, kEpiMulWeight, false>(g, grid, st);
-    case kEpiGatedSilu:
-      return packed ? launch_one<DT, BM, kEpiGatedSilu, true>(g, grid, st)
-                    : launch_one<DT, BM, kEpiGatedSilu, false>(g, grid, st);
-    default:
-      return packed ? launch_one<DT, BM, kEpiPlain, true>(g, grid, st)
-                    : launch_one<DT, BM, kEpiPlain, false>(g, grid, st);
+    case kEpiMulWeight: return launch_one<DT, BM, kEpiMulWeight>(g, grid, st);
+    case kEpiGatedSilu: return launch_one<DT, BM, kEpiGatedSilu>(g, grid, st);
+    default: return launch_one<DT, BM, kEpiPlain>(g, grid, st);
   }
 }
 
 // Entry used by sarathi_moe_grouped_gemm; block_m is 64, 128 or 256.  `g` is complete except
 // for n_blocks, which depends on the epilogue.
-int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, bool packed,
-                        int dtype, hipStream_t st) {
+int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, int dtype,
+                        hipStream_t st) {
   const int64_t cols_per_block = epilogue == kEpiGatedSilu ? 128 : 256;
   g.n_blocks = (int32_t)((out_cols + cols_per_block - 1) / cols_per_block);
   const int64_t blocks = (int64_t)((g.n_blocks + 7) / 8) * g.m_blocks * 8;
@@ -319,9 +293,9 @@ int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int block_m, int epilog
   const dim3 grid((unsigned)blocks);
 #define SK_PICK(DT)                                                                      \
   switch (block_m) {                                                                     \
-    case 64: return launch_epilogue<DT, 64>(g, grid, epilogue, packed, st);              \
-    case 128: return launch_epilogue<DT, 128>(g, grid, epilogue, packed, st);            \
-    default: return launch_epilogue<DT, 256>(g, grid, epilogue, packed, st);             \
+    case 64: return launch_epilogue<DT, 64>(g, grid, epilogue, st);              \
+    case 128: return launch_epilogue<DT, 128>(g, grid, epilogue, st);            \
+    default: return launch_epilogue<DT, 256>(g, grid, epilogue, st);             \
   }
   if (dtype == kBF16) { SK_PICK(kBF16) } else { SK_PICK(kF16) }
 #undef SK_PICK
