@@ -219,7 +219,7 @@ int sarathi_fused_topk_align(float* topk_weights, int32_t* topk_indices,
  * order the matrix cores consume them: per expert ceil(N/32) row tiles, each
  * K/16 blocks of 1 KiB, a block holding for lane l = (n mod 32) + 32*((k mod 16)/8)
  * the 8 elements k mod 8 = 0..7 (rows beyond N zero); b_expert_stride then
- * counts ceil(N/32)*32*K elements.  Same results, 1.1-1.25x faster.
+ * counts ceil(N/32)*32*K elements.  Same results, 1.1-1.2x faster.
  */
 #define SARATHI_MOE_B_ROW_MAJOR 0
 #define SARATHI_MOE_B_PACKED 1

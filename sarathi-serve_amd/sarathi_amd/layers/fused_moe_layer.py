@@ -59,7 +59,7 @@ class FusedMoE(torch.nn.Module):
 
     def pack_weights(self, inplace: bool = False) -> None:
         """Re-tile both weight tensors once, after loading, into the order the grouped GEMM's
-        matrix-core loads consume (1.1-1.25x faster GEMMs, same results).  By default this keeps a
+        matrix-core loads consume (1.1-1.2x faster GEMMs, same results).  By default this keeps a
         second copy of the weights; ``inplace=True`` re-tiles inside the parameters' own storage
         (no extra memory; the parameters then hold the packed values).  Call again after changing
         the weights."""
