@@ -47,6 +47,9 @@ def _close(got, want, what):
     (40, 8, 2, 256, 300, 128, False),    # mostly padding
     (33, 16, 4, 32, 256, 64, True),      # some experts empty, single K step
     (5, 8, 1, 32, 1024, 192, False),
+    (600, 8, 2, 32, 256, 128, True),     # 45 slot blocks
+    (1200, 8, 2, 64, 520, 128, False),   # many blocks through both kernels' 64-slot variants, ragged N
+    (2100, 4, 2, 128, 256, 64, True),    # 36 blocks of 128
 ])
 def test_grouped_gemm_matches_formulation(ops, dev, dtype, T, E, k, BM, N, K, mul):
     _, w, ids, s, e, p = _route(T, E, k, BM, T + N)
