@@ -11,7 +11,8 @@
 //
 // Tiling: a workgroup of four waves owns BM slots x 256 output columns; wave w
 // owns columns [64 w, 64 w + 64) for all BM slots, as 32x32 MFMA tiles
-// (v_mfma_f32_32x32x16 bf16 / f16, 16 deep).  The MFMA "A" operand is fed with
+// (v_mfma_f32_32x32x16 bf16 / f16, 16 deep).  (BM = 256: eight waves, two rows
+// of four, 128 slots per row.)  The MFMA "A" operand is fed with
 // WEIGHT rows and the "B" operand with TOKEN rows, so a lane ends up holding
 // four consecutive output columns of one token per accumulator quad and the
 // epilogue writes 8-byte pieces of C rows.
@@ -22,7 +23,9 @@
 //            of their use, with no second register buffer.  Two layouts of B:
 //              row-major [E, N, K] (the reference's): a wave's operand load
 //                touches 32 rows x 32 bytes, which makes the texture-address
-//                unit, not the MFMA pipe, the limit (~22-36 % of peak);
+//                unit, not the MFMA pipe, the limit (~22-36 % of peak); only
+//                32-slot blocks take this path, larger ones run the kernel of
+//                moe_gemm_lds.hip;
 //              packed    [E, N/32, K/16, 64 lanes, 8]: the 1 KiB a wave needs for
 //                one 32x16 operand is contiguous in lane order, one fully
 //                coalesced load (~1.3-1.9x faster in this kernel).  Weights are static, so
@@ -37,9 +40,11 @@
 // its two weight tiles, so gate and up of an output element sit in the same lane, and
 // C [slots, N/2] = T(T(silu(T(gate))) * T(up)) is written directly: bit-identical to the
 // unfused pair of kernels, without the [slots, N] intermediate ever reaching memory.
+// 32-slot tiles of a block that hold only padding are skipped.
 // Workgroup ids are mapped so that the eight XCDs (id mod 8) each take their
-// own column blocks and walk the slot blocks fastest: workgroups that run
-// together on an XCD share the expert's weight tile in that XCD's L2.
+// own column blocks, four of them side by side over all slot blocks: workgroups
+// that run together on an XCD share token tiles and the experts' weight tiles
+// in that XCD's L2 (tile_of_block).
 #include "moe_gemm_common.h"
 #include "launch.h"
 

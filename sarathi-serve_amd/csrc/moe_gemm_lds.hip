@@ -20,6 +20,7 @@
 //            32 KiB per K-step.
 // LDS: 2 x (BM x 128 bytes of tokens + 32 KiB of weights), 128 KiB at BM = 256, requested as dynamic
 // shared memory.
+#include <atomic>
 #include "moe_gemm_common.h"
 #include "launch.h"
 
@@ -260,14 +261,14 @@ static int launch_one(const MoeGemmArgs& g, dim3 grid, hipStream_t st) {
   auto kernel = moe_gemm_lds_kernel<DT, BM, EPI>;
   constexpr int bytes = lds_bytes(BM);
   // more LDS than the default per-workgroup limit: opt in once per kernel and device
-  static bool raised[64] = {};
+  static std::atomic<bool> raised[64] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return SARATHI_ERR_LAUNCH;
-  if (!raised[dev]) {
+  if (!raised[dev].load(std::memory_order_acquire)) {  // racing first calls both set it: harmless
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
       return SARATHI_ERR_LAUNCH;
-    raised[dev] = true;
+    raised[dev].store(true, std::memory_order_release);
   }
   hipLaunchKernelGGL(kernel, grid, dim3(64 * kLdsWaves), bytes, st, g);
   return launch_status();

@@ -81,10 +81,11 @@ def get_default_config(M: int, E: int, N: int, K: int, topk: int, dtype: Optiona
                        packed: bool = True) -> Dict[str, int]:
     """Slot-block size for M tokens: the more slots an expert receives, the taller the tile (a
     taller tile re-uses each weight fragment for more tokens).  Thresholds from sweeps of the
-    Mixtral-8x7B shape on MI355X (tune_fused_moe.py): with packed weights 256 is never the
-    fastest; row-major weights are fastest through the kernel that shares both operands in LDS
-    (blocks of 64 and more), with 256-slot blocks from ~100 slots per expert.  BLOCK_SIZE_N / BLOCK_SIZE_K are fixed properties of the kernel, reported for
-    information."""
+    Mixtral-8x7B shape on MI355X (tune_fused_moe.py): with packed weights 128 and 256 are within
+    a few per cent of each other at large batches (the tuned tables pick per batch size);
+    row-major weights are fastest through the kernel that shares both operands in LDS (blocks of
+    64 and more), with 256-slot blocks from ~100 slots per expert.  BLOCK_SIZE_N / BLOCK_SIZE_K
+    are fixed properties of the kernel, reported for information."""
     per_expert = M * topk / max(E, 1)
     if not packed:   # row-major weights run the LDS kernel, which starts at 64-slot blocks
         block_m = 256 if per_expert >= 96 else 128 if per_expert >= 48 else 64
