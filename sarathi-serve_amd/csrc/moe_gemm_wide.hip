@@ -1,0 +1,301 @@
+// Grouped expert GEMM for row-major ([E, N, K]) expert weights at 256-slot blocks: four waves,
+// one per SIMD, each owning a 128 x 128 accumulator tile.
+//
+// Same computation and argument block as moe_gemm.hip / moe_gemm_lds.hip.  The eight-wave LDS
+// kernel moves every operand byte global -> LDS with buffer loads that write LDS directly; those
+// can only be issued once every wave has finished reading the buffer they overwrite, so all 64
+// of a K-step's transfers leave in one burst behind the barrier, the vector-memory front end
+// backs up, and the MFMAs queued behind them wait (removing the transfers from that loop: +28 %;
+// feeding them cache-resident data instead: only +9 %).  Here the operands pass through
+// registers: a thread's 16 global loads of K-step i + 2 are spread over K-step i, stay in
+// registers for one K-step, and are stored to LDS during K-step i + 1 (see the loop): loads and
+// LDS stores trickle out between the MFMAs instead of piling up behind a barrier.  That takes 64
+// registers on top of 256 accumulators and 64 of operand fragments, hence one wave per SIMD
+// with the full 512-entry register file, and a 128 x 128 wave tile, which also needs a third
+// fewer LDS bytes per flop than 128 x 64.
+//
+// LDS: two buffers of (256 token rows + 256 weight rows) x 128 bytes, the 16-byte chunks of a
+// row rotated as in the other kernels (bank-conflict-free operand reads); 128 KiB, requested as
+// dynamic shared memory.
+#include <atomic>
+#include "moe_gemm_common.h"
+#include "launch.h"
+
+namespace sarathi_hip {
+
+constexpr int kWideUnits = 256 * 8;                      // 16-byte units of one operand buffer
+constexpr int kWideLdsBytes = 2 * 2 * kWideUnits * 16;   // tokens + weights, double buffered
+
+template <int DT, int EPI>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void moe_gemm_wide_kernel(MoeGemmArgs g) {
+  constexpr bool MUL_WEIGHT = EPI == kEpiMulWeight;
+  constexpr bool GATED = EPI == kEpiGatedSilu;
+  constexpr int BM = 256, BN = 256;
+  constexpr int MT = 4, NT = 4, SUB = kGemmBK / 16;
+  constexpr int ROWS = 8;  // rows of each operand a thread moves per K-step
+  extern __shared__ u32x4 lds[];
+  u32x4* const tok = lds;                   // [2][256 rows][8 units]
+  u32x4* const wgt = lds + 2 * kWideUnits;  // [2][256 rows][8 units]
+
+  int pid_m, pid_n;
+  if (!tile_of_block(g, blockIdx.x, pid_m, pid_n)) return;
+  if (pid_m * BM >= *g.num_tokens_post_padded) return;
+  const int expert = g.expert_ids[pid_m];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wc = wave & 1;                 // wave column: 128 weight rows
+  const int row0 = (wave >> 1) * (BM / 2);  // wave row: first slot of this wave inside the block
+  const int l32 = lane & 31, grp = lane >> 5;
+  const int half_n = g.N >> 1;  // gated: weight rows [half_n, N) are the up projection
+
+  // Row R of the workgroup's weight tile -> row of the expert's matrix, or -1 beyond it.  Gated:
+  // a wave column holds 64 gate rows (tiles 0, 1) and the 64 matching up rows (tiles 2, 3), so
+  // gate and up of an output element end up in the same lane.
+  auto weight_row = [&](int R) {
+    if constexpr (GATED) {
+      const int gate = pid_n * (BN / 2) + (R >> 7) * 64 + ((R >> 5) & 1) * 32 + (R & 31);
+      return gate < half_n ? gate + ((R >> 6) & 1) * half_n : -1;
+    } else {
+      const int n = pid_n * BN + R;
+      return n < g.N ? n : -1;
+    }
+  };
+
+  // ---- global -> register -> LDS: thread t moves position t & 7 of rows (t >> 3) + 32 j
+  const rsrc_t ra = make_rsrc(g.a, g.a_bytes);
+  const rsrc_t rb = make_rsrc(reinterpret_cast<const char*>(g.b) + (int64_t)expert * g.b_expert_stride * 2,
+                              (uint32_t)((int64_t)g.N * g.K * 2));
+  const int pos = tid & 7;
+  uint32_t a_off[ROWS], w_off[ROWS];
+#pragma unroll
+  for (int j = 0; j < ROWS; ++j) {
+    const int r = (tid >> 3) + 32 * j;
+    const uint32_t chunk = (uint32_t)lds_chunk_at(r, pos) * 16u;
+    const int slot_index = pid_m * BM + r;
+    const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
+    // a padding slot reads beyond the end of A, i.e. zeros, whatever K offset is added
+    a_off[j] = sid < g.num_valid ? (uint32_t)(sid / g.top_k) * (uint32_t)(g.a_row_stride * 2) + chunk
+                                 : g.a_bytes;
+    const int n = weight_row(r);
+    w_off[j] = n >= 0 ? (uint32_t)n * (uint32_t)g.K * 2u + chunk : 0x80000000u;
+  }
+  u32x4 st_tok[ROWS], st_wgt[ROWS];  // one K-step of operands on its way from global memory to LDS
+  auto load_rows = [&](int k0, u32x4 (&t)[ROWS], u32x4 (&w)[ROWS], int j0, int j1) {
+#pragma unroll
+    for (int j = j0; j < j1; ++j) {
+      t[j] = buf_load16<kCached>(ra, a_off[j] + (uint32_t)k0 * 2u);
+      w[j] = buf_load16<kCached>(rb, w_off[j] + (uint32_t)k0 * 2u);
+    }
+  };
+  auto store_rows = [&](int buf, const u32x4 (&t)[ROWS], const u32x4 (&w)[ROWS], int j0, int j1) {
+#pragma unroll
+    for (int j = j0; j < j1; ++j) {
+      const int unit = ((tid >> 3) + 32 * j) * 8 + pos;
+      tok[buf * kWideUnits + unit] = t[j];
+      wgt[buf * kWideUnits + unit] = w[j];
+    }
+  };
+
+  f32x16 acc[NT][MT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[nt][mt][i] = 0.f;
+
+  // tiles of 32 slots without a valid slot are skipped (see moe_gemm.hip)
+  int mt_live = 0;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int slot_index = pid_m * BM + row0 + mt * 32 + l32;
+    const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
+    if (__ballot(sid < g.num_valid) != 0ull) mt_live = mt + 1;
+  }
+
+  const int steps = g.K / kGemmBK;
+  auto wrap = [&](int k) { return k < steps ? k : k - steps; };  // k < 2 * steps
+  // K-step j is read from LDS buffer j & 1
+  load_rows(0, st_tok, st_wgt, 0, ROWS);
+  store_rows(0, st_tok, st_wgt, 0, ROWS);
+  load_rows(wrap(1) * kGemmBK, st_tok, st_wgt, 0, ROWS);
+  lds_barrier();
+
+  // During K-step i (LDS buffer i & 1 is read), row by row of a thread's share:
+  //   sub-steps 0..2  store the registers, which hold K-step i + 1 since they were loaded during
+  //                   K-step i - 1, to the other LDS buffer, which nobody reads since the last
+  //                   barrier, and load K-step i + 2 into them (the last loads in sub-step 3);
+  //   before sub-step 3  barrier: the stores above are visible and every wave has read all it
+  //                   needs of this buffer (sub-step 3's operands are in registers already), so
+  //                   the first operands of K-step i + 1 are read under sub-step 3's MFMAs.
+  // Branch-free: the last two K-steps load and store wrapped-around data that is never used.
+  auto k_loop = [&](auto live_tag) {
+    constexpr int LIVE = decltype(live_tag)::value;  // token tiles 0 .. LIVE - 1 are computed
+    auto read_operands = [&](int buf, int s, u32x4 (&tv)[MT], u32x4 (&wv)[NT]) {
+      const u32x4* tb = tok + buf * kWideUnits;
+      const u32x4* wb = wgt + buf * kWideUnits;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        if (mt >= LIVE) continue;
+        const int r = row0 + mt * 32 + l32;
+        tv[mt] = tb[r * 8 + lds_slot(r, 2 * s + grp)];
+      }
+      if (LIVE == 0) return;
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const int R = wc * 128 + nt * 32 + l32;
+        wv[nt] = wb[R * 8 + lds_slot(R, 2 * s + grp)];
+      }
+    };
+    u32x4 tv[2][MT], wv[2][NT];
+    read_operands(0, 0, tv[0], wv[0]);
+    auto sub_step = [&](auto s_tag, int cur, int k_load) {
+      constexpr int s = decltype(s_tag)::value;
+      constexpr int ST0 = s * 3, ST1 = s * 3 + 3 < ROWS ? s * 3 + 3 : ROWS;  // rows stored here
+      if constexpr (s + 1 < SUB) {
+        read_operands(cur, s + 1, tv[(s + 1) & 1], wv[(s + 1) & 1]);
+        store_rows(cur ^ 1, st_tok, st_wgt, ST0, ST1);
+      } else {
+        lds_barrier();
+        read_operands(cur ^ 1, 0, tv[0], wv[0]);
+      }
+      // rows 0-1, 2-3, 4-5, 6-7: each after its store (rows 0-2, 3-5, 6-7).  (Loading every row
+      // right after its store, for a full K-step between load and store, crowds the first two
+      // sub-steps with memory instructions and measured 2.5 % slower.)
+      load_rows(k_load, st_tok, st_wgt, s * 2, s * 2 + 2);
+      if constexpr (LIVE == 0) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          if (mt >= LIVE) continue;
+          acc[nt][mt] = mfma32<DT>(wv[s & 1][nt], tv[s & 1][mt], acc[nt][mt]);
+        }
+      if constexpr (LIVE == MT) {
+        // One wave per SIMD: nothing else runs while this wave issues memory instructions, so
+        // they go out one at a time in the shadow of the MFMAs (each MFMA keeps the matrix
+        // core busy for 32 cycles): 8 LDS reads, the LDS stores, then the global loads.  (Measured
+        // against: the compiler's own order, 7 % slower; stores and loads ahead of the reads,
+        // 4 % slower; reads two per MFMA, equal.)
+        constexpr int kMfma = 0x008, kVmemRead = 0x020, kDsRead = 0x100, kDsWrite = 0x200;
+        constexpr int WRITES = s + 1 < SUB ? 2 * (ST1 - ST0) : 0;
+#pragma unroll
+        for (int i = 0; i < MT + NT; ++i) {
+          __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < WRITES; ++i) {
+          __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(kDsWrite, 1, 0);
+        }
+        // the four global loads over the MFMAs that are left (2, 2, 4, 8)
+        constexpr int LEFT = MT * NT - (MT + NT) - WRITES;
+        constexpr int PER = LEFT >= 4 ? 1 : 2;
+#pragma unroll
+        for (int i = 0; i < 4 / PER; ++i) {
+          __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(kVmemRead, PER, 0);
+        }
+      } else if constexpr (LIVE > 0) {
+        // partly filled blocks: the same idea with fewer MFMAs to hide behind
+        constexpr int kMfma = 0x008, kMemory = 0x020 | 0x100 | 0x200;
+        constexpr int OPS = LIVE + NT + (s + 1 < SUB ? 2 * (ST1 - ST0) : 0) + 4;
+        constexpr int PER = (OPS + NT * LIVE - 1) / (NT * LIVE);
+#pragma unroll
+        for (int i = 0; i < NT * LIVE; ++i) {
+          __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(kMemory, PER, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    for (int step = 0; step < steps; ++step) {
+      const int cur = step & 1;
+      const int k_load = wrap(wrap(step + 1) + 1) * kGemmBK;  // K-step step + 2
+      sub_step(std::integral_constant<int, 0>{}, cur, k_load);
+      sub_step(std::integral_constant<int, 1>{}, cur, k_load);
+      sub_step(std::integral_constant<int, 2>{}, cur, k_load);
+      sub_step(std::integral_constant<int, 3>{}, cur, k_load);
+    }
+  };
+  call_with_live<MT>(mt_live, k_loop);
+
+  // ---- epilogue: lane holds, per accumulator quad, 4 consecutive columns of one token
+  const int n_wave0 = GATED ? pid_n * (BN / 2) + wc * 64 : pid_n * BN + wc * 128;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int slot_index = pid_m * BM + row0 + mt * 32 + l32;
+    const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
+    if (sid >= g.num_valid) continue;
+    float scale = 1.f;
+    if constexpr (MUL_WEIGHT) scale = g.topk_weights[sid];
+    char* crow = reinterpret_cast<char*>(g.c) + (int64_t)sid * g.c_row_stride * 2;
+    constexpr int OUT_TILES = GATED ? NT / 2 : NT;
+#pragma unroll
+    for (int nt = 0; nt < OUT_TILES; ++nt) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n_wave0 + nt * 32 + q * 8 + grp * 4;
+        const int n_end = GATED ? half_n : g.N;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if constexpr (GATED) {
+            const float x = rnd<DT>(acc[nt][mt][q * 4 + e]), y = rnd<DT>(acc[nt + 2][mt][q * 4 + e]);
+            v[e] = rnd<DT>(silu_f32(x)) * y;
+          } else {
+            v[e] = acc[nt][mt][q * 4 + e];
+            if constexpr (MUL_WEIGHT) v[e] *= scale;
+          }
+        }
+        if (n + 3 < n_end) {
+          u32x2 out = {pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
+          *reinterpret_cast<u32x2*>(crow + (int64_t)n * 2) = out;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < n_end) store_elem<DT>(crow, n + e, v[e]);
+        }
+      }
+    }
+  }
+}
+
+template <int DT, int EPI>
+static int launch_wide(const MoeGemmArgs& g, dim3 grid, hipStream_t st) {
+  auto kernel = moe_gemm_wide_kernel<DT, EPI>;
+  // more LDS than the default per-workgroup limit: opt in once per kernel and device
+  static std::atomic<bool> raised[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return SARATHI_ERR_LAUNCH;
+  if (!raised[dev].load(std::memory_order_acquire)) {  // racing first calls both set it: harmless
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kWideLdsBytes) != hipSuccess)
+      return SARATHI_ERR_LAUNCH;
+    raised[dev].store(true, std::memory_order_release);
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(256), kWideLdsBytes, st, g);
+  return launch_status();
+}
+
+// Entry used by sarathi_moe_grouped_gemm for row-major weights at 256-slot blocks.  `g` is
+// complete except for n_blocks, which depends on the epilogue.
+int launch_moe_gemm_wide(MoeGemmArgs g, int64_t out_cols, int epilogue, int dtype, hipStream_t st) {
+  const int64_t cols_per_block = epilogue == kEpiGatedSilu ? 128 : 256;
+  g.n_blocks = (int32_t)((out_cols + cols_per_block - 1) / cols_per_block);
+  const int64_t blocks = (int64_t)((g.n_blocks + 7) / 8) * g.m_blocks * 8;
+  if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)blocks);
+#define SK_PICK(DT)                                                         \
+  switch (epilogue) {                                                       \
+    case kEpiMulWeight: return launch_wide<DT, kEpiMulWeight>(g, grid, st); \
+    case kEpiGatedSilu: return launch_wide<DT, kEpiGatedSilu>(g, grid, st); \
+    default: return launch_wide<DT, kEpiPlain>(g, grid, st);                \
+  }
+  if (dtype == kBF16) { SK_PICK(kBF16) } else { SK_PICK(kF16) }
+#undef SK_PICK
+}
+
+}  // namespace sarathi_hip
