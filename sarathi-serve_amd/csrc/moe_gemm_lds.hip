@@ -1,5 +1,5 @@
 // Grouped expert GEMM for row-major ([E, N, K]) expert weights, both operands through LDS, at
-// block sizes 64, 128 and 256.
+// block sizes 64 and 128 (256-slot blocks run the four-wave kernel of moe_gemm_wide.hip).
 //
 // Same computation and argument block as moe_gemm.hip.  That kernel feeds the weights from global
 // memory straight into registers, wave by wave: with the packed layout every such load is one
@@ -7,8 +7,8 @@
 // or more apart, and the vector-memory front end becomes the limit.  Here a workgroup of EIGHT
 // waves owns BM slots x 256 output columns: two wave rows of BM / 2 slots share each weight
 // tile, and four wave columns share each token tile, both through LDS, so a compute unit loads
-// 64 KB per 64-deep K-step for 8.4 MFLOP (BM = 256).  Every wave holds a (BM / 2) x 64
-// accumulator tile (128 registers at BM = 256), so two waves fit on a SIMD.
+// 48 KB per 64-deep K-step for 4.2 MFLOP at BM = 128.  Every wave holds a (BM / 2) x 64
+// accumulator tile (64 registers at BM = 128).
 //
 // Data movement: every global -> LDS transfer is a buffer load that writes LDS directly (no
 // register staging), issued one K-step ahead into the other half of a double buffer; one barrier
@@ -18,7 +18,7 @@
 //   weights  a strip's 64 rows x 128 bytes are fetched as whole 128-byte row segments (eight
 //            lanes per row: fully coalesced) into the same rotated row layout as the tokens;
 //            32 KiB per K-step.
-// LDS: 2 x (BM x 128 bytes of tokens + 32 KiB of weights), 128 KiB at BM = 256, requested as dynamic
+// LDS: 2 x (BM x 128 bytes of tokens + 32 KiB of weights), 96 KiB at BM = 128, requested as dynamic
 // shared memory.
 #include <atomic>
 #include "moe_gemm_common.h"
@@ -31,8 +31,7 @@ constexpr int kLdsWgtUnits = 256 * 8;  // 16-byte units of a weight buffer (256 
 // dynamic shared memory of a workgroup with BM slots: tokens + weights, double buffered
 constexpr int lds_bytes(int BM) { return 2 * (BM * 8 + kLdsWgtUnits) * 16; }
 
-// BM = 256 (two waves per SIMD, 128 KiB of LDS: one workgroup per compute unit) is the large-batch
-// shape; BM = 64 and 128 exist for row-major weights at small batches, where the coalesced
+// BM = 64 and 128: row-major weights at small and medium batches, where the coalesced
 // row-segment fetch is what matters and several workgroups share a compute unit.
 template <int DT, int BM, int EPI>
 __global__ __launch_bounds__(64 * kLdsWaves) __attribute__((amdgpu_waves_per_eu(2)))
@@ -283,7 +282,7 @@ static int launch_epilogue(const MoeGemmArgs& g, dim3 grid, int epilogue, hipStr
   }
 }
 
-// Entry used by sarathi_moe_grouped_gemm; block_m is 64, 128 or 256.  `g` is complete except
+// Entry used by sarathi_moe_grouped_gemm; block_m is 64 or 128.  `g` is complete except
 // for n_blocks, which depends on the epilogue.
 int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, int dtype,
                         hipStream_t st) {
@@ -295,8 +294,7 @@ int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int block_m, int epilog
 #define SK_PICK(DT)                                                                      \
   switch (block_m) {                                                                     \
     case 64: return launch_epilogue<DT, 64>(g, grid, epilogue, st);              \
-    case 128: return launch_epilogue<DT, 128>(g, grid, epilogue, st);            \
-    default: return launch_epilogue<DT, 256>(g, grid, epilogue, st);             \
+    default: return launch_epilogue<DT, 128>(g, grid, epilogue, st);             \
   }
   if (dtype == kBF16) { SK_PICK(kBF16) } else { SK_PICK(kF16) }
 #undef SK_PICK
