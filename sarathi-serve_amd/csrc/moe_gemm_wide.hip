@@ -23,20 +23,27 @@
 
 namespace sarathi_hip {
 
-constexpr int kWideUnits = 256 * 8;                      // 16-byte units of one operand buffer
-constexpr int kWideLdsBytes = 2 * 2 * kWideUnits * 16;   // tokens + weights, double buffered
+constexpr int kWideUnits = 256 * 8;  // 16-byte units of a token buffer (256 rows x 128 bytes)
+// dynamic shared memory: tokens + BN weight rows, double buffered
+constexpr int wide_lds_bytes(int BN) { return 2 * (kWideUnits + BN * 8) * 16; }
 
-template <int DT, int EPI>
+// BN = 256 is the shape described above.  BN = 128 (wave tiles of 128 x 64) exists for launches
+// that would otherwise have too few workgroups to keep every compute unit streaming weights:
+// the down projection of a decode-size batch is 8 experts x 16 column blocks of 256.
+template <int DT, int EPI, int BN>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void moe_gemm_wide_kernel(MoeGemmArgs g) {
   constexpr bool MUL_WEIGHT = EPI == kEpiMulWeight;
   constexpr bool GATED = EPI == kEpiGatedSilu;
-  constexpr int BM = 256, BN = 256;
-  constexpr int MT = 4, NT = 4, SUB = kGemmBK / 16;
-  constexpr int ROWS = 8;  // rows of each operand a thread moves per K-step
+  constexpr int BM = 256;
+  constexpr int MT = 4, NT = BN / 64, SUB = kGemmBK / 16;
+  constexpr int WCR = BN / 2;      // weight rows of a wave column
+  constexpr int ROWS = 8;          // token rows a thread moves per K-step
+  constexpr int W_ROWS = BN / 32;  // weight rows a thread moves per K-step
+  constexpr int kWgtUnits = BN * 8;
   extern __shared__ u32x4 lds[];
   u32x4* const tok = lds;                   // [2][256 rows][8 units]
-  u32x4* const wgt = lds + 2 * kWideUnits;  // [2][256 rows][8 units]
+  u32x4* const wgt = lds + 2 * kWideUnits;  // [2][BN rows][8 units]
 
   int pid_m, pid_n;
   if (!tile_of_block(g, blockIdx.x, pid_m, pid_n)) return;
@@ -44,18 +51,19 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
   const int expert = g.expert_ids[pid_m];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wc = wave & 1;                 // wave column: 128 weight rows
+  const int wc = wave & 1;                 // wave column: BN / 2 weight rows
   const int row0 = (wave >> 1) * (BM / 2);  // wave row: first slot of this wave inside the block
   const int l32 = lane & 31, grp = lane >> 5;
   const int half_n = g.N >> 1;  // gated: weight rows [half_n, N) are the up projection
 
   // Row R of the workgroup's weight tile -> row of the expert's matrix, or -1 beyond it.  Gated:
-  // a wave column holds 64 gate rows (tiles 0, 1) and the 64 matching up rows (tiles 2, 3), so
-  // gate and up of an output element end up in the same lane.
+  // the first half of a wave column's tiles are gate rows and the second half the matching up
+  // rows, so gate and up of an output element end up in the same lane.
   auto weight_row = [&](int R) {
     if constexpr (GATED) {
-      const int gate = pid_n * (BN / 2) + (R >> 7) * 64 + ((R >> 5) & 1) * 32 + (R & 31);
-      return gate < half_n ? gate + ((R >> 6) & 1) * half_n : -1;
+      const int in_col = R % WCR;  // row inside the wave column
+      const int gate = pid_n * (BN / 2) + (R / WCR) * (WCR / 2) + in_col % (WCR / 2);
+      return gate < half_n ? gate + (in_col / (WCR / 2)) * half_n : -1;
     } else {
       const int n = pid_n * BN + R;
       return n < g.N ? n : -1;
@@ -67,7 +75,7 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
   const rsrc_t rb = make_rsrc(reinterpret_cast<const char*>(g.b) + (int64_t)expert * g.b_expert_stride * 2,
                               (uint32_t)((int64_t)g.N * g.K * 2));
   const int pos = tid & 7;
-  uint32_t a_off[ROWS], w_off[ROWS];
+  uint32_t a_off[ROWS], w_off[W_ROWS];
 #pragma unroll
   for (int j = 0; j < ROWS; ++j) {
     const int r = (tid >> 3) + 32 * j;
@@ -77,23 +85,27 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
     // a padding slot reads beyond the end of A, i.e. zeros, whatever K offset is added
     a_off[j] = sid < g.num_valid ? (uint32_t)(sid / g.top_k) * (uint32_t)(g.a_row_stride * 2) + chunk
                                  : g.a_bytes;
-    const int n = weight_row(r);
-    w_off[j] = n >= 0 ? (uint32_t)n * (uint32_t)g.K * 2u + chunk : 0x80000000u;
+    if (j < W_ROWS) {
+      const int n = weight_row(r);
+      w_off[j] = n >= 0 ? (uint32_t)n * (uint32_t)g.K * 2u + chunk : 0x80000000u;
+    }
   }
-  u32x4 st_tok[ROWS], st_wgt[ROWS];  // one K-step of operands on its way from global memory to LDS
-  auto load_rows = [&](int k0, u32x4 (&t)[ROWS], u32x4 (&w)[ROWS], int j0, int j1) {
+  // one K-step of operands on its way from global memory to LDS; row j of both operands (the
+  // weights have rows j < W_ROWS only) moves together
+  u32x4 st_tok[ROWS], st_wgt[W_ROWS];
+  auto load_rows = [&](int k0, int j0, int j1) {
 #pragma unroll
     for (int j = j0; j < j1; ++j) {
-      t[j] = buf_load16<kCached>(ra, a_off[j] + (uint32_t)k0 * 2u);
-      w[j] = buf_load16<kCached>(rb, w_off[j] + (uint32_t)k0 * 2u);
+      st_tok[j] = buf_load16<kCached>(ra, a_off[j] + (uint32_t)k0 * 2u);
+      if (j < W_ROWS) st_wgt[j] = buf_load16<kCached>(rb, w_off[j] + (uint32_t)k0 * 2u);
     }
   };
-  auto store_rows = [&](int buf, const u32x4 (&t)[ROWS], const u32x4 (&w)[ROWS], int j0, int j1) {
+  auto store_rows = [&](int buf, int j0, int j1) {
 #pragma unroll
     for (int j = j0; j < j1; ++j) {
       const int unit = ((tid >> 3) + 32 * j) * 8 + pos;
-      tok[buf * kWideUnits + unit] = t[j];
-      wgt[buf * kWideUnits + unit] = w[j];
+      tok[buf * kWideUnits + unit] = st_tok[j];
+      if (j < W_ROWS) wgt[buf * kWgtUnits + unit] = st_wgt[j];
     }
   };
 
@@ -117,9 +129,9 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
   const int steps = g.K / kGemmBK;
   auto wrap = [&](int k) { return k < steps ? k : k - steps; };  // k < 2 * steps
   // K-step j is read from LDS buffer j & 1
-  load_rows(0, st_tok, st_wgt, 0, ROWS);
-  store_rows(0, st_tok, st_wgt, 0, ROWS);
-  load_rows(wrap(1) * kGemmBK, st_tok, st_wgt, 0, ROWS);
+  load_rows(0, 0, ROWS);
+  store_rows(0, 0, ROWS);
+  load_rows(wrap(1) * kGemmBK, 0, ROWS);
   lds_barrier();
 
   // During K-step i (LDS buffer i & 1 is read), row by row of a thread's share:
@@ -134,7 +146,7 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
     constexpr int LIVE = decltype(live_tag)::value;  // token tiles 0 .. LIVE - 1 are computed
     auto read_operands = [&](int buf, int s, u32x4 (&tv)[MT], u32x4 (&wv)[NT]) {
       const u32x4* tb = tok + buf * kWideUnits;
-      const u32x4* wb = wgt + buf * kWideUnits;
+      const u32x4* wb = wgt + buf * kWgtUnits;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         if (mt >= LIVE) continue;
@@ -144,7 +156,7 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
       if (LIVE == 0) return;
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-        const int R = wc * 128 + nt * 32 + l32;
+        const int R = wc * WCR + nt * 32 + l32;
         wv[nt] = wb[R * 8 + lds_slot(R, 2 * s + grp)];
       }
     };
@@ -155,7 +167,7 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
       constexpr int ST0 = s * 3, ST1 = s * 3 + 3 < ROWS ? s * 3 + 3 : ROWS;  // rows stored here
       if constexpr (s + 1 < SUB) {
         read_operands(cur, s + 1, tv[(s + 1) & 1], wv[(s + 1) & 1]);
-        store_rows(cur ^ 1, st_tok, st_wgt, ST0, ST1);
+        store_rows(cur ^ 1, ST0, ST1);
       } else {
         lds_barrier();
         read_operands(cur ^ 1, 0, tv[0], wv[0]);
@@ -163,7 +175,7 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
       // rows 0-1, 2-3, 4-5, 6-7: each after its store (rows 0-2, 3-5, 6-7).  (Loading every row
       // right after its store, for a full K-step between load and store, crowds the first two
       // sub-steps with memory instructions and measured 2.5 % slower.)
-      load_rows(k_load, st_tok, st_wgt, s * 2, s * 2 + 2);
+      load_rows(k_load, s * 2, s * 2 + 2);
       if constexpr (LIVE == 0) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
@@ -172,7 +184,7 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
           if (mt >= LIVE) continue;
           acc[nt][mt] = mfma32<DT>(wv[s & 1][nt], tv[s & 1][mt], acc[nt][mt]);
         }
-      if constexpr (LIVE == MT) {
+      if constexpr (LIVE == MT && BN == 256) {
         // One wave per SIMD: nothing else runs while this wave issues memory instructions, so
         // they go out one at a time in the shadow of the MFMAs (each MFMA keeps the matrix
         // core busy for 32 cycles): 8 LDS reads, the LDS stores, then the global loads.  (Measured
@@ -199,9 +211,13 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
           __builtin_amdgcn_sched_group_barrier(kVmemRead, PER, 0);
         }
       } else if constexpr (LIVE > 0) {
-        // partly filled blocks: the same idea with fewer MFMAs to hide behind
+        // partly filled blocks, narrow column blocks: the same idea with fewer MFMAs to hide
+        // behind (several memory instructions per MFMA)
         constexpr int kMfma = 0x008, kMemory = 0x020 | 0x100 | 0x200;
-        constexpr int OPS = LIVE + NT + (s + 1 < SUB ? 2 * (ST1 - ST0) : 0) + 4;
+        constexpr int W0 = ST0 < W_ROWS ? ST0 : W_ROWS, W1 = ST1 < W_ROWS ? ST1 : W_ROWS;
+        constexpr int STORES = s + 1 < SUB ? (ST1 - ST0) + (W1 - W0) : 0;
+        constexpr int L0 = s * 2 < W_ROWS ? s * 2 : W_ROWS, L1 = s * 2 + 2 < W_ROWS ? s * 2 + 2 : W_ROWS;
+        constexpr int OPS = LIVE + NT + STORES + 2 + (L1 - L0);
         constexpr int PER = (OPS + NT * LIVE - 1) / (NT * LIVE);
 #pragma unroll
         for (int i = 0; i < NT * LIVE; ++i) {
@@ -223,7 +239,7 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
   call_with_live<MT>(mt_live, k_loop);
 
   // ---- epilogue: lane holds, per accumulator quad, 4 consecutive columns of one token
-  const int n_wave0 = GATED ? pid_n * (BN / 2) + wc * 64 : pid_n * BN + wc * 128;
+  const int n_wave0 = GATED ? pid_n * (BN / 2) + wc * (WCR / 2) : pid_n * BN + wc * WCR;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int slot_index = pid_m * BM + row0 + mt * 32 + l32;
@@ -243,7 +259,7 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           if constexpr (GATED) {
-            const float x = rnd<DT>(acc[nt][mt][q * 4 + e]), y = rnd<DT>(acc[nt + 2][mt][q * 4 + e]);
+            const float x = rnd<DT>(acc[nt][mt][q * 4 + e]), y = rnd<DT>(acc[nt + NT / 2][mt][q * 4 + e]);
             v[e] = rnd<DT>(silu_f32(x)) * y;
           } else {
             v[e] = acc[nt][mt][q * 4 + e];
@@ -263,39 +279,52 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
   }
 }
 
-template <int DT, int EPI>
+template <int DT, int EPI, int BN>
 static int launch_wide(const MoeGemmArgs& g, dim3 grid, hipStream_t st) {
-  auto kernel = moe_gemm_wide_kernel<DT, EPI>;
+  auto kernel = moe_gemm_wide_kernel<DT, EPI, BN>;
+  constexpr int bytes = wide_lds_bytes(BN);
   // more LDS than the default per-workgroup limit: opt in once per kernel and device
   static std::atomic<bool> raised[64] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return SARATHI_ERR_LAUNCH;
   if (!raised[dev].load(std::memory_order_acquire)) {  // racing first calls both set it: harmless
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kWideLdsBytes) != hipSuccess)
+                            hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
       return SARATHI_ERR_LAUNCH;
     raised[dev].store(true, std::memory_order_release);
   }
-  hipLaunchKernelGGL(kernel, grid, dim3(256), kWideLdsBytes, st, g);
+  hipLaunchKernelGGL(kernel, grid, dim3(256), bytes, st, g);
   return launch_status();
 }
 
-// Entry used by sarathi_moe_grouped_gemm for row-major weights at 256-slot blocks.  `g` is
-// complete except for n_blocks, which depends on the epilogue.
-int launch_moe_gemm_wide(MoeGemmArgs g, int64_t out_cols, int epilogue, int dtype, hipStream_t st) {
-  const int64_t cols_per_block = epilogue == kEpiGatedSilu ? 128 : 256;
+template <int DT, int BN>
+static int launch_wide_epilogue(MoeGemmArgs g, int64_t out_cols, int epilogue, hipStream_t st) {
+  const int64_t cols_per_block = epilogue == kEpiGatedSilu ? BN / 2 : BN;
   g.n_blocks = (int32_t)((out_cols + cols_per_block - 1) / cols_per_block);
   const int64_t blocks = (int64_t)((g.n_blocks + 7) / 8) * g.m_blocks * 8;
   if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)blocks);
-#define SK_PICK(DT)                                                         \
-  switch (epilogue) {                                                       \
-    case kEpiMulWeight: return launch_wide<DT, kEpiMulWeight>(g, grid, st); \
-    case kEpiGatedSilu: return launch_wide<DT, kEpiGatedSilu>(g, grid, st); \
-    default: return launch_wide<DT, kEpiPlain>(g, grid, st);                \
+  switch (epilogue) {
+    case kEpiMulWeight: return launch_wide<DT, kEpiMulWeight, BN>(g, grid, st);
+    case kEpiGatedSilu: return launch_wide<DT, kEpiGatedSilu, BN>(g, grid, st);
+    default: return launch_wide<DT, kEpiPlain, BN>(g, grid, st);
   }
-  if (dtype == kBF16) { SK_PICK(kBF16) } else { SK_PICK(kF16) }
-#undef SK_PICK
+}
+
+// Entry used by sarathi_moe_grouped_gemm for row-major weights at 256-slot blocks.  `g` is
+// complete except for n_blocks, which depends on the epilogue and the column-block width.
+int launch_moe_gemm_wide(MoeGemmArgs g, int64_t out_cols, int epilogue, int dtype, hipStream_t st) {
+  // column blocks of 256 unless that leaves compute units without a workgroup (measured on the
+  // Mixtral down projection: 128-wide blocks are 1-12 % faster up to 512 tokens, where the wide
+  // launch has 128-192 workgroups, and 20 % slower from 1024 tokens on, where it has 256)
+  const int64_t cols_wide = epilogue == kEpiGatedSilu ? 128 : 256;
+  const int64_t wide_blocks = (out_cols + cols_wide - 1) / cols_wide * g.m_blocks;
+  const bool narrow = wide_blocks < 256;
+  if (dtype == kBF16)
+    return narrow ? launch_wide_epilogue<kBF16, 128>(g, out_cols, epilogue, st)
+                  : launch_wide_epilogue<kBF16, 256>(g, out_cols, epilogue, st);
+  return narrow ? launch_wide_epilogue<kF16, 128>(g, out_cols, epilogue, st)
+                : launch_wide_epilogue<kF16, 256>(g, out_cols, epilogue, st);
 }
 
 }  // namespace sarathi_hip

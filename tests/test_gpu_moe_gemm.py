@@ -50,6 +50,8 @@ def _close(got, want, what):
     (600, 8, 2, 32, 256, 128, True),     # 45 slot blocks
     (1200, 8, 2, 64, 520, 128, False),   # many blocks through both kernels' 64-slot variants, ragged N
     (2100, 4, 2, 128, 256, 64, True),    # 36 blocks of 128
+    (1500, 4, 2, 256, 4100, 128, True),  # 16 slot blocks x 17 column blocks: the 256-wide tiles of
+                                         # the four-wave kernel (smaller launches take 128-wide ones)
 ])
 def test_grouped_gemm_matches_formulation(ops, dev, dtype, T, E, k, BM, N, K, mul):
     _, w, ids, s, e, p = _route(T, E, k, BM, T + N)
@@ -239,6 +241,7 @@ def test_fused_moe_module(ops, dev, grouped):
     (1000, 8, 2, 128, 640, 128),     # I not a multiple of the 128 output columns of a workgroup
     (40, 4, 2, 256, 96, 64),
     (77, 4, 1, 32, 20, 64),          # I = 20: row-major only (packed tiles would straddle)
+    (1500, 4, 2, 256, 2080, 64),     # enough workgroups for the four-wave kernel's 256-wide tiles
 ])
 def test_gated_silu_epilogue_is_bit_identical_to_separate_kernels(ops, dev, dtype, T, E, k, BM, I, K):
     _, w, ids, s, e, p = _route(T, E, k, BM, T + I)
