@@ -216,8 +216,11 @@ void moe_gemm_kernel(MoeGemmArgs g) {
         // of the next sub-step ahead of its MFMAs
         __builtin_amdgcn_sched_barrier(0);
       }
-      // the DMA of this step is older than the NT * SUB weight loads issued since
-      wait_vmcnt<NT * SUB>();
+      // the DMA of this step is older than the NT * SUB weight loads issued since.  A wave
+      // without live tiles (eight-wave variant: a wave row that is all padding) has no use for
+      // its weight loads, so the compiler drops them: it must wait for everything, or its share
+      // of the token gather could still be in flight when the others pass the barrier.
+      wait_vmcnt<LIVE == 0 ? 0 : NT * SUB>();
       lds_barrier();
     }
   };

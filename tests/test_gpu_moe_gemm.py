@@ -111,6 +111,37 @@ def test_grouped_gemm_padding_anywhere_in_a_block(ops, dev, BM, packed):
     assert torch.equal(outs[0], outs[1])
 
 
+@pytest.mark.parametrize("packed", [False, True])
+def test_grouped_gemm_half_empty_256_blocks_repeatable(ops, dev, packed):
+    """256-slot blocks in which the second wave row holds only padding: those waves compute
+    nothing but still move their share of the operands and must not let the others pass a
+    barrier before it has landed (a wait sized for loads that the compiler had dropped once let
+    them).  Many K-steps, many repetitions, every result identical and equal to the formulation."""
+    T, E, k, BM, N, K = 60, 8, 2, 256, 512, 1536
+    _, w, ids, s, e, p = _route(T, E, k, BM, 77)
+    assert int(torch.bincount(ids.flatten().long(), minlength=E).max()) <= 128
+    g = gen(78)
+    A = randn((T, K), g, std=0.5)
+    Bw = randn((E, N, K), g, std=0.5)
+    want = torch.zeros((T, k, N), dtype=torch.bfloat16)
+    torch_formulations.moe_grouped_gemm(A, Bw, want, w, s, e, p, T * k, BM, k, False)
+    Bd = Bw.to(dev)
+    if packed:
+        from sarathi_amd.layers import pack_expert_weights
+        Bd = pack_expert_weights(Bd).data
+    args = (A.to(dev), Bd)
+    tail = (w.to(dev), s.to(dev), e.to(dev), p.to(dev), T * k, BM, k, False, packed, N)
+    first = None
+    for rep in range(40):
+        got = torch.full((T, k, N), 7.0, dtype=torch.bfloat16, device=dev)
+        ops.moe_ops.moe_grouped_gemm(*args, got, *tail)
+        if first is None:
+            first = got
+            _close(first, want, "half-empty blocks")
+        else:
+            assert torch.equal(got, first), "repetition %d differs" % rep
+
+
 def test_grouped_gemm_second_stage_addressing(ops, dev):
     """top_k = 1 addressing of the down projection: A rows are slots (tokens * topk of them)."""
     T, E, k, BM, N, K = 200, 8, 2, 64, 256, 128
