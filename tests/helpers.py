@@ -68,6 +68,9 @@ def assert_close_dtype(got, want, atol=1e-2, rtol=1e-2, max_ulps=2, max_mismatch
         ulp = torch.maximum(ulp_of(got), ulp_of(want))[fin]
         ulps = (diff / ulp)[bad].max().item()
         assert ulps <= max_ulps + 1e-3, "max error %.2f ulp" % ulps
-    # the fraction is a statistical bound: a tiny tensor may hold a couple of one-ulp flips
-    assert frac <= max(max_mismatch_frac, 2.0 / diff.numel()), "mismatching fraction %.3g" % frac
+    # the fraction is a statistical bound: for n elements that each flip with probability
+    # max_mismatch_frac, allow the mean count plus four standard deviations plus two
+    n = diff.numel()
+    allowed = max_mismatch_frac * n + 4.0 * (max_mismatch_frac * n) ** 0.5 + 2.0
+    assert int(bad.sum()) <= allowed, "mismatching fraction %.3g (%d of %d)" % (frac, int(bad.sum()), n)
     return frac
