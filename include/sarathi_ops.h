@@ -219,8 +219,8 @@ int sarathi_fused_topk_align(float* topk_weights, int32_t* topk_indices,
  * order the matrix cores consume them: per expert ceil(N/32) row tiles, each
  * K/16 blocks of 1 KiB, a block holding for lane l = (n mod 32) + 32*((k mod 16)/8)
  * the 8 elements k mod 8 = 0..7 (rows beyond N zero); b_expert_stride then
- * counts ceil(N/32)*32*K elements.  Same results; up to 1.15x
- * faster at small batches, within a few per cent of row-major at large ones.
+ * counts ceil(N/32)*32*K elements.  Same results; within a few
+ * per cent of the row-major path at every batch size.
  */
 #define SARATHI_MOE_B_ROW_MAJOR 0
 #define SARATHI_MOE_B_PACKED 1

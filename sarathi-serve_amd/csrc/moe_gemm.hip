@@ -305,8 +305,9 @@ static int launch_moe_gemm(const MoeGemmArgs& g, int epilogue, bool packed, hipS
 // moe_gemm_lds.hip: row-major weights, both operands shared through LDS
 int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, int dtype,
                         hipStream_t st);
-// moe_gemm_wide.hip: row-major weights at 256-slot blocks, four waves with 128 x 128 tiles
-int launch_moe_gemm_wide(MoeGemmArgs g, int64_t out_cols, int epilogue, int dtype, hipStream_t st);
+// moe_gemm_wide.hip: row-major weights at 64- and 256-slot blocks, four waves
+int launch_moe_gemm_wide(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, int dtype,
+                         hipStream_t st);
 
 }  // namespace sarathi_hip
 
@@ -373,10 +374,12 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
   g.group_n = kGemmGroupN;
   hipStream_t st = (hipStream_t)stream;
   const int mw = epilogue;
-  // row-major weights: 256-slot blocks run the four-wave kernel with 128 x 128 wave tiles
-  if (!packed && block_m == 256) return launch_moe_gemm_wide(g, c_cols, mw, dtype, st);
-  // ... 64- and 128-slot blocks the eight-wave kernel with both operands through LDS
-  if (!packed && block_m >= 64) return launch_moe_gemm_lds(g, c_cols, block_m, mw, dtype, st);
+  // row-major weights: 256- and 64-slot blocks run the four-wave kernel (128 x 128 wave tiles
+  // for large batches, 32-slot wave tiles for decode-size ones)
+  if (!packed && (block_m == 256 || block_m == 64))
+    return launch_moe_gemm_wide(g, c_cols, block_m, mw, dtype, st);
+  // ... 128-slot blocks the eight-wave kernel with both operands through LDS
+  if (!packed && block_m == 128) return launch_moe_gemm_lds(g, c_cols, block_m, mw, dtype, st);
 #define SK_GEMM(DT)                                                       \
   switch (block_m) {                                                      \
     case 32: return launch_moe_gemm<DT, 32>(g, mw, packed, st);           \

@@ -1,5 +1,5 @@
 // Grouped expert GEMM for row-major ([E, N, K]) expert weights, both operands through LDS, at
-// block sizes 64 and 128 (256-slot blocks run the four-wave kernel of moe_gemm_wide.hip).
+// 128-slot blocks (64- and 256-slot blocks run the four-wave kernel of moe_gemm_wide.hip).
 //
 // Same computation and argument block as moe_gemm.hip.  That kernel feeds the weights from global
 // memory straight into registers, wave by wave: with the packed layout every such load is one
@@ -31,8 +31,7 @@ constexpr int kLdsWgtUnits = 256 * 8;  // 16-byte units of a weight buffer (256 
 // dynamic shared memory of a workgroup with BM slots: tokens + weights, double buffered
 constexpr int lds_bytes(int BM) { return 2 * (BM * 8 + kLdsWgtUnits) * 16; }
 
-// BM = 64 and 128: row-major weights at small and medium batches, where the coalesced
-// row-segment fetch is what matters and several workgroups share a compute unit.
+// BM = 128 is the block size in use (the kernel body is generic in BM = 64, 128, 256).
 template <int DT, int BM, int EPI>
 __global__ __launch_bounds__(64 * kLdsWaves) __attribute__((amdgpu_waves_per_eu(2)))
 void moe_gemm_lds_kernel(MoeGemmArgs g) {
@@ -282,7 +281,7 @@ static int launch_epilogue(const MoeGemmArgs& g, dim3 grid, int epilogue, hipStr
   }
 }
 
-// Entry used by sarathi_moe_grouped_gemm; block_m is 64 or 128.  `g` is complete except
+// Entry used by sarathi_moe_grouped_gemm; block_m is 128.  `g` is complete except
 // for n_blocks, which depends on the epilogue.
 int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, int dtype,
                         hipStream_t st) {
@@ -291,11 +290,8 @@ int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int block_m, int epilog
   const int64_t blocks = (int64_t)((g.n_blocks + 7) / 8) * g.m_blocks * 8;
   if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)blocks);
-#define SK_PICK(DT)                                                                      \
-  switch (block_m) {                                                                     \
-    case 64: return launch_epilogue<DT, 64>(g, grid, epilogue, st);              \
-    default: return launch_epilogue<DT, 128>(g, grid, epilogue, st);             \
-  }
+#define SK_PICK(DT) return launch_epilogue<DT, 128>(g, grid, epilogue, st);
+  (void)block_m;
   if (dtype == kBF16) { SK_PICK(kBF16) } else { SK_PICK(kF16) }
 #undef SK_PICK
 }

@@ -23,27 +23,29 @@
 
 namespace sarathi_hip {
 
-constexpr int kWideUnits = 256 * 8;  // 16-byte units of a token buffer (256 rows x 128 bytes)
-// dynamic shared memory: tokens + BN weight rows, double buffered
-constexpr int wide_lds_bytes(int BN) { return 2 * (kWideUnits + BN * 8) * 16; }
+// dynamic shared memory: BM token rows + BN weight rows of 128 bytes, double buffered
+constexpr int wide_lds_bytes(int BM, int BN) { return 2 * (BM * 8 + BN * 8) * 16; }
 
 // BN = 256 is the shape described above.  BN = 128 (wave tiles of 128 x 64) exists for launches
 // that would otherwise have too few workgroups to keep every compute unit streaming weights:
 // the down projection of a decode-size batch is 8 experts x 16 column blocks of 256.
-template <int DT, int EPI, int BN>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+// BM = 64 (wave tiles of 32 slots x BN / 2 columns, 64 or 32 accumulator registers, 48-80 KiB of
+// LDS) is the same loop for decode-size batches: two or three workgroups share a compute unit, so
+// that more weight bytes are in flight while nearly all the time goes into streaming them.
+template <int DT, int EPI, int BN, int BM>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, BM == 256 ? 1 : 4)))
 void moe_gemm_wide_kernel(MoeGemmArgs g) {
   constexpr bool MUL_WEIGHT = EPI == kEpiMulWeight;
   constexpr bool GATED = EPI == kEpiGatedSilu;
-  constexpr int BM = 256;
-  constexpr int MT = 4, NT = BN / 64, SUB = kGemmBK / 16;
+  constexpr int MT = BM / 64, NT = BN / 64, SUB = kGemmBK / 16;
   constexpr int WCR = BN / 2;      // weight rows of a wave column
-  constexpr int ROWS = 8;          // token rows a thread moves per K-step
+  constexpr int ROWS = 8;          // rows of an operand a thread moves per K-step, at most
+  constexpr int T_ROWS = BM / 32;  // token rows a thread moves per K-step
   constexpr int W_ROWS = BN / 32;  // weight rows a thread moves per K-step
-  constexpr int kWgtUnits = BN * 8;
+  constexpr int kTokUnits = BM * 8, kWgtUnits = BN * 8;
   extern __shared__ u32x4 lds[];
-  u32x4* const tok = lds;                   // [2][256 rows][8 units]
-  u32x4* const wgt = lds + 2 * kWideUnits;  // [2][BN rows][8 units]
+  u32x4* const tok = lds;                  // [2][BM rows][8 units]
+  u32x4* const wgt = lds + 2 * kTokUnits;  // [2][BN rows][8 units]
 
   int pid_m, pid_n;
   if (!tile_of_block(g, blockIdx.x, pid_m, pid_n)) return;
@@ -75,28 +77,30 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
   const rsrc_t rb = make_rsrc(reinterpret_cast<const char*>(g.b) + (int64_t)expert * g.b_expert_stride * 2,
                               (uint32_t)((int64_t)g.N * g.K * 2));
   const int pos = tid & 7;
-  uint32_t a_off[ROWS], w_off[W_ROWS];
+  uint32_t a_off[T_ROWS], w_off[W_ROWS];
 #pragma unroll
   for (int j = 0; j < ROWS; ++j) {
     const int r = (tid >> 3) + 32 * j;
     const uint32_t chunk = (uint32_t)lds_chunk_at(r, pos) * 16u;
-    const int slot_index = pid_m * BM + r;
-    const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
-    // a padding slot reads beyond the end of A, i.e. zeros, whatever K offset is added
-    a_off[j] = sid < g.num_valid ? (uint32_t)(sid / g.top_k) * (uint32_t)(g.a_row_stride * 2) + chunk
-                                 : g.a_bytes;
+    if (j < T_ROWS) {
+      const int slot_index = pid_m * BM + r;
+      const int sid = slot_index < g.em ? g.sorted_token_ids[slot_index] : g.num_valid;
+      // a padding slot reads beyond the end of A, i.e. zeros, whatever K offset is added
+      a_off[j] = sid < g.num_valid ? (uint32_t)(sid / g.top_k) * (uint32_t)(g.a_row_stride * 2) + chunk
+                                   : g.a_bytes;
+    }
     if (j < W_ROWS) {
       const int n = weight_row(r);
       w_off[j] = n >= 0 ? (uint32_t)n * (uint32_t)g.K * 2u + chunk : 0x80000000u;
     }
   }
-  // one K-step of operands on its way from global memory to LDS; row j of both operands (the
-  // weights have rows j < W_ROWS only) moves together
-  u32x4 st_tok[ROWS], st_wgt[W_ROWS];
+  // one K-step of operands on its way from global memory to LDS; row j of both operands (as
+  // far as each has a row j) moves together
+  u32x4 st_tok[T_ROWS], st_wgt[W_ROWS];
   auto load_rows = [&](int k0, int j0, int j1) {
 #pragma unroll
     for (int j = j0; j < j1; ++j) {
-      st_tok[j] = buf_load16<kCached>(ra, a_off[j] + (uint32_t)k0 * 2u);
+      if (j < T_ROWS) st_tok[j] = buf_load16<kCached>(ra, a_off[j] + (uint32_t)k0 * 2u);
       if (j < W_ROWS) st_wgt[j] = buf_load16<kCached>(rb, w_off[j] + (uint32_t)k0 * 2u);
     }
   };
@@ -104,7 +108,7 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
 #pragma unroll
     for (int j = j0; j < j1; ++j) {
       const int unit = ((tid >> 3) + 32 * j) * 8 + pos;
-      tok[buf * kWideUnits + unit] = st_tok[j];
+      if (j < T_ROWS) tok[buf * kTokUnits + unit] = st_tok[j];
       if (j < W_ROWS) wgt[buf * kWgtUnits + unit] = st_wgt[j];
     }
   };
@@ -145,7 +149,7 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
   auto k_loop = [&](auto live_tag) {
     constexpr int LIVE = decltype(live_tag)::value;  // token tiles 0 .. LIVE - 1 are computed
     auto read_operands = [&](int buf, int s, u32x4 (&tv)[MT], u32x4 (&wv)[NT]) {
-      const u32x4* tb = tok + buf * kWideUnits;
+      const u32x4* tb = tok + buf * kTokUnits;
       const u32x4* wb = wgt + buf * kWgtUnits;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
@@ -184,7 +188,7 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
           if (mt >= LIVE) continue;
           acc[nt][mt] = mfma32<DT>(wv[s & 1][nt], tv[s & 1][mt], acc[nt][mt]);
         }
-      if constexpr (LIVE == MT && BN == 256) {
+      if constexpr (LIVE == MT && BN == 256 && BM == 256) {
         // One wave per SIMD: nothing else runs while this wave issues memory instructions, so
         // they go out one at a time in the shadow of the MFMAs (each MFMA keeps the matrix
         // core busy for 32 cycles): 8 LDS reads, the LDS stores, then the global loads.  (Measured
@@ -214,10 +218,12 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
         // partly filled blocks, narrow column blocks: the same idea with fewer MFMAs to hide
         // behind (several memory instructions per MFMA)
         constexpr int kMfma = 0x008, kMemory = 0x020 | 0x100 | 0x200;
-        constexpr int W0 = ST0 < W_ROWS ? ST0 : W_ROWS, W1 = ST1 < W_ROWS ? ST1 : W_ROWS;
-        constexpr int STORES = s + 1 < SUB ? (ST1 - ST0) + (W1 - W0) : 0;
-        constexpr int L0 = s * 2 < W_ROWS ? s * 2 : W_ROWS, L1 = s * 2 + 2 < W_ROWS ? s * 2 + 2 : W_ROWS;
-        constexpr int OPS = LIVE + NT + STORES + 2 + (L1 - L0);
+        constexpr auto rows_in = [](int j0, int j1, int n) {  // rows j0 <= j < j1 that are below n
+          return (j1 < n ? j1 : n) - (j0 < n ? j0 : n);
+        };
+        constexpr int STORES = s + 1 < SUB ? rows_in(ST0, ST1, T_ROWS) + rows_in(ST0, ST1, W_ROWS) : 0;
+        constexpr int LOADS = rows_in(s * 2, s * 2 + 2, T_ROWS) + rows_in(s * 2, s * 2 + 2, W_ROWS);
+        constexpr int OPS = LIVE + NT + STORES + LOADS;
         constexpr int PER = (OPS + NT * LIVE - 1) / (NT * LIVE);
 #pragma unroll
         for (int i = 0; i < NT * LIVE; ++i) {
@@ -279,10 +285,10 @@ void moe_gemm_wide_kernel(MoeGemmArgs g) {
   }
 }
 
-template <int DT, int EPI, int BN>
+template <int DT, int EPI, int BN, int BM>
 static int launch_wide(const MoeGemmArgs& g, dim3 grid, hipStream_t st) {
-  auto kernel = moe_gemm_wide_kernel<DT, EPI, BN>;
-  constexpr int bytes = wide_lds_bytes(BN);
+  auto kernel = moe_gemm_wide_kernel<DT, EPI, BN, BM>;
+  constexpr int bytes = wide_lds_bytes(BM, BN);
   // more LDS than the default per-workgroup limit: opt in once per kernel and device
   static std::atomic<bool> raised[64] = {};
   int dev = 0;
@@ -297,7 +303,7 @@ static int launch_wide(const MoeGemmArgs& g, dim3 grid, hipStream_t st) {
   return launch_status();
 }
 
-template <int DT, int BN>
+template <int DT, int BN, int BM>
 static int launch_wide_epilogue(MoeGemmArgs g, int64_t out_cols, int epilogue, hipStream_t st) {
   const int64_t cols_per_block = epilogue == kEpiGatedSilu ? BN / 2 : BN;
   g.n_blocks = (int32_t)((out_cols + cols_per_block - 1) / cols_per_block);
@@ -305,26 +311,33 @@ static int launch_wide_epilogue(MoeGemmArgs g, int64_t out_cols, int epilogue, h
   if (blocks > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)blocks);
   switch (epilogue) {
-    case kEpiMulWeight: return launch_wide<DT, kEpiMulWeight, BN>(g, grid, st);
-    case kEpiGatedSilu: return launch_wide<DT, kEpiGatedSilu, BN>(g, grid, st);
-    default: return launch_wide<DT, kEpiPlain, BN>(g, grid, st);
+    case kEpiMulWeight: return launch_wide<DT, kEpiMulWeight, BN, BM>(g, grid, st);
+    case kEpiGatedSilu: return launch_wide<DT, kEpiGatedSilu, BN, BM>(g, grid, st);
+    default: return launch_wide<DT, kEpiPlain, BN, BM>(g, grid, st);
   }
 }
 
-// Entry used by sarathi_moe_grouped_gemm for row-major weights at 256-slot blocks.  `g` is
-// complete except for n_blocks, which depends on the epilogue and the column-block width.
-int launch_moe_gemm_wide(MoeGemmArgs g, int64_t out_cols, int epilogue, int dtype, hipStream_t st) {
-  // column blocks of 256 unless that leaves compute units without a workgroup (measured on the
-  // Mixtral down projection: 128-wide blocks are 1-12 % faster up to 512 tokens, where the wide
-  // launch has 128-192 workgroups, and 20 % slower from 1024 tokens on, where it has 256)
+// Entry used by sarathi_moe_grouped_gemm for row-major weights at 64- and 256-slot blocks.  `g`
+// is complete except for n_blocks, which depends on the epilogue and the column-block width.
+int launch_moe_gemm_wide(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, int dtype,
+                         hipStream_t st) {
+  // Column blocks of 256 unless that leaves compute units short of workgroups.  Measured on the
+  // Mixtral projections: at 256-slot blocks (one workgroup per compute unit) 128-wide blocks are
+  // 1-12 % faster while the wide launch has fewer than 256 workgroups and 20 % slower from there
+  // on; at 64-slot blocks (two to three per compute unit) they are faster up to 896 workgroups
+  // (16-64 tokens: gate/up projection 0.333 -> 0.326 ms, down projection 0.205 -> 0.178 ms) and
+  // slower at 1792 (256 tokens).
   const int64_t cols_wide = epilogue == kEpiGatedSilu ? 128 : 256;
   const int64_t wide_blocks = (out_cols + cols_wide - 1) / cols_wide * g.m_blocks;
-  const bool narrow = wide_blocks < 256;
-  if (dtype == kBF16)
-    return narrow ? launch_wide_epilogue<kBF16, 128>(g, out_cols, epilogue, st)
-                  : launch_wide_epilogue<kBF16, 256>(g, out_cols, epilogue, st);
-  return narrow ? launch_wide_epilogue<kF16, 128>(g, out_cols, epilogue, st)
-                : launch_wide_epilogue<kF16, 256>(g, out_cols, epilogue, st);
+  const bool narrow = wide_blocks < (block_m == 256 ? 256 : 1024);
+#define SK_PICK(DT)                                                                               \
+  if (block_m == 256)                                                                             \
+    return narrow ? launch_wide_epilogue<DT, 128, 256>(g, out_cols, epilogue, st)                 \
+                  : launch_wide_epilogue<DT, 256, 256>(g, out_cols, epilogue, st);                \
+  return narrow ? launch_wide_epilogue<DT, 128, 64>(g, out_cols, epilogue, st)                    \
+                : launch_wide_epilogue<DT, 256, 64>(g, out_cols, epilogue, st);
+  if (dtype == kBF16) { SK_PICK(kBF16) } else { SK_PICK(kF16) }
+#undef SK_PICK
 }
 
 }  // namespace sarathi_hip

@@ -24,8 +24,8 @@ class PackedExpertWeights:
     """Expert weights [E, N, K] re-tiled once into the order the matrix cores consume them
     (see ``pack_expert_weights``).  Pass it wherever ``fused_moe`` / ``fused_experts`` /
     ``invoke_fused_moe_kernel`` take ``w1`` / ``w2`` / ``B``; results are the same as with the
-    row-major tensor; the grouped GEMM runs up to 1.15x faster at small batches (weight
-    streaming) and within a few per cent of the row-major path at large ones."""
+    row-major tensor and the grouped GEMM runs within a few per cent of the row-major path
+    (faster or slower, by batch size), so packing is optional."""
 
     def __init__(self, data: torch.Tensor, shape):
         self.data = data                      # [E, ceil(N/32), K/16, 2, 32, 8]
@@ -84,17 +84,13 @@ def get_default_config(M: int, E: int, N: int, K: int, topk: int, dtype: Optiona
     taller tile re-uses each weight fragment for more tokens).  Thresholds from sweeps of the
     Mixtral-8x7B, Mixtral-8x22B and a 64-expert shape on MI355X (tune_fused_moe.py): with packed
     weights 128 and 256 are within a few per cent of each other at large batches (the tuned
-    tables pick per batch size); with row-major weights the 256-slot kernel (four waves, 128 x 128
-    tiles) is the fastest from ~100 slots per expert on, and with few experts at every batch size,
-    down to single tokens (it streams the weights best); with many experts and few slots each
-    the eight-wave LDS kernel at 64 or 128 slots wastes less on padding.  BLOCK_SIZE_N /
-    BLOCK_SIZE_K are fixed properties of the kernel, reported for information."""
+    tables pick per batch size); row-major weights run the four-wave kernel, with 64-slot blocks
+    (small tiles, several workgroups per compute unit: weight streaming) up to ~64 slots per expert
+    and 256-slot blocks (128 x 128 wave tiles) beyond, a little later with many experts.
+    BLOCK_SIZE_N / BLOCK_SIZE_K are fixed properties of the kernels, reported for information."""
     per_expert = M * topk / max(E, 1)
-    if not packed:   # row-major weights: blocks of 64 and more
-        if per_expert >= 96 or E <= 16:
-            block_m = 256
-        else:
-            block_m = 128 if per_expert >= 48 else 64
+    if not packed:
+        block_m = 256 if per_expert >= (64 if E <= 16 else 128) else 64
     else:
         block_m = 128 if per_expert >= 48 else 64 if per_expert >= 10 else 32
     return {"BLOCK_SIZE_M": block_m, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 64, "GROUP_SIZE_M": 1}

@@ -59,8 +59,8 @@ class FusedMoE(torch.nn.Module):
 
     def pack_weights(self, inplace: bool = False) -> None:
         """Re-tile both weight tensors once, after loading, into the order the grouped GEMM's
-        matrix-core loads consume (same results; up to 1.15x faster GEMMs at small batches, within
-        a few per cent of the row-major path at large ones).  By default this keeps a
+        matrix-core loads consume (same results; within a few per cent of the row-major path at every
+        batch size, so this is optional).  By default this keeps a
         second copy of the weights; ``inplace=True`` re-tiles inside the parameters' own storage
         (no extra memory; the parameters then hold the packed values).  Call again after changing
         the weights."""
