@@ -25,7 +25,7 @@
 //                touches 32 rows x 32 bytes, which makes the texture-address
 //                unit, not the MFMA pipe, the limit (~22-36 % of peak); only
 //                32-slot blocks take this path, larger ones run the kernel of
-//                moe_gemm_lds.hip;
+//                moe_gemm_wide.hip;
 //              packed    [E, N/32, K/16, 64 lanes, 8]: the 1 KiB a wave needs for
 //                one 32x16 operand is contiguous in lane order, one fully
 //                coalesced load (~1.3-1.9x faster in this kernel).  Weights are static, so
@@ -302,10 +302,7 @@ static int launch_moe_gemm(const MoeGemmArgs& g, int epilogue, bool packed, hipS
   return launch_status();
 }
 
-// moe_gemm_lds.hip: row-major weights, both operands shared through LDS
-int launch_moe_gemm_lds(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, int dtype,
-                        hipStream_t st);
-// moe_gemm_wide.hip: row-major weights at 64- and 256-slot blocks, four waves
+// moe_gemm_wide.hip: row-major weights at 64-, 128- and 256-slot blocks, four waves
 int launch_moe_gemm_wide(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, int dtype,
                          hipStream_t st);
 
@@ -374,12 +371,9 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
   g.group_n = kGemmGroupN;
   hipStream_t st = (hipStream_t)stream;
   const int mw = epilogue;
-  // row-major weights: 256- and 64-slot blocks run the four-wave kernel (128 x 128 wave tiles
-  // for large batches, 32-slot wave tiles for decode-size ones)
-  if (!packed && (block_m == 256 || block_m == 64))
-    return launch_moe_gemm_wide(g, c_cols, block_m, mw, dtype, st);
-  // ... 128-slot blocks the eight-wave kernel with both operands through LDS
-  if (!packed && block_m == 128) return launch_moe_gemm_lds(g, c_cols, block_m, mw, dtype, st);
+  // row-major weights run the four-wave kernel of moe_gemm_wide.hip from 64-slot blocks on (32-slot
+  // wave tiles for decode-size batches, 128 x 128 wave tiles at 256-slot blocks)
+  if (!packed && block_m >= 64) return launch_moe_gemm_wide(g, c_cols, block_m, mw, dtype, st);
 #define SK_GEMM(DT)                                                       \
   switch (block_m) {                                                      \
     case 32: return launch_moe_gemm<DT, 32>(g, mw, packed, st);           \

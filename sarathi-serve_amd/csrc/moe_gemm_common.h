@@ -1,4 +1,4 @@
-// Pieces shared by the grouped expert GEMM kernels (moe_gemm.hip, moe_gemm_lds.hip).
+// Pieces shared by the grouped expert GEMM kernels (moe_gemm.hip, moe_gemm_wide.hip).
 #pragma once
 
 #include <stdint.h>

@@ -1,22 +1,27 @@
-// Grouped expert GEMM for row-major ([E, N, K]) expert weights at 256-slot blocks: four waves,
-// one per SIMD, each owning a 128 x 128 accumulator tile.
+// Grouped expert GEMM for row-major ([E, N, K]) expert weights: four waves, one per SIMD at
+// 256-slot blocks, each owning a 128 x 128 accumulator tile (smaller tiles at 64- and 128-slot
+// blocks).
 //
-// Same computation and argument block as moe_gemm.hip / moe_gemm_lds.hip.  The eight-wave LDS
-// kernel moves every operand byte global -> LDS with buffer loads that write LDS directly; those
-// can only be issued once every wave has finished reading the buffer they overwrite, so all 64
-// of a K-step's transfers leave in one burst behind the barrier, the vector-memory front end
-// backs up, and the MFMAs queued behind them wait (removing the transfers from that loop: +28 %;
-// feeding them cache-resident data instead: only +9 %).  Here the operands pass through
-// registers: a thread's 16 global loads of K-step i + 2 are spread over K-step i, stay in
-// registers for one K-step, and are stored to LDS during K-step i + 1 (see the loop): loads and
-// LDS stores trickle out between the MFMAs instead of piling up behind a barrier.  That takes 64
-// registers on top of 256 accumulators and 64 of operand fragments, hence one wave per SIMD
-// with the full 512-entry register file, and a 128 x 128 wave tile, which also needs a third
-// fewer LDS bytes per flop than 128 x 64.
+// Same computation and argument block as moe_gemm.hip.  That kernel feeds the weights from global
+// memory straight into registers, wave by wave: with the packed layout every such load is one
+// contiguous KiB, but with row-major weights a lane's 16 bytes come from 32 different rows, 8 KB
+// or more apart.  Here both operands are shared through LDS and fetched as whole 128-byte row
+// segments (eight lanes per row).  An earlier kernel moved them global -> LDS with buffer loads
+// that write LDS directly, eight waves per workgroup; such a transfer can only be issued once
+// every wave has finished reading the buffer it overwrites, so all 64 of a K-step's transfers
+// left in one burst behind the barrier, the vector-memory front end backed up, and the MFMAs
+// queued behind them waited (removing the transfers from that loop: +28 %; feeding them
+// cache-resident data instead: only +9 %).  Here the operands pass through registers: a thread's
+// 16 global loads of K-step i + 2 are spread over K-step i, stay in registers for one K-step, and
+// are stored to LDS during K-step i + 1 (see the loop): loads and LDS stores trickle out between
+// the MFMAs instead of piling up behind a barrier.  That takes 64 registers on top of 256
+// accumulators and 64 of operand fragments, hence one wave per SIMD with the full 512-entry
+// register file, and a 128 x 128 wave tile, which also needs a third fewer LDS bytes per flop
+// than 128 x 64.
 //
-// LDS: two buffers of (256 token rows + 256 weight rows) x 128 bytes, the 16-byte chunks of a
-// row rotated as in the other kernels (bank-conflict-free operand reads); 128 KiB, requested as
-// dynamic shared memory.
+// LDS: two buffers of (BM token rows + BN weight rows) x 128 bytes, the 16-byte chunks of a row
+// rotated as in moe_gemm.hip (bank-conflict-free operand reads); 128 KiB at BM = BN = 256,
+// requested as dynamic shared memory.
 #include <atomic>
 #include "moe_gemm_common.h"
 #include "launch.h"
@@ -32,8 +37,9 @@ constexpr int wide_lds_bytes(int BM, int BN) { return 2 * (BM * 8 + BN * 8) * 16
 // BM = 64 (wave tiles of 32 slots x BN / 2 columns, 64 or 32 accumulator registers, 48-80 KiB of
 // LDS) is the same loop for decode-size batches: two or three workgroups share a compute unit, so
 // that more weight bytes are in flight while nearly all the time goes into streaming them.
+// BM = 128 (64-slot wave tiles) completes the set of block sizes.
 template <int DT, int EPI, int BN, int BM>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, BM == 256 ? 1 : 4)))
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, BM == 256 ? 1 : BM == 128 ? 2 : 4)))
 void moe_gemm_wide_kernel(MoeGemmArgs g) {
   constexpr bool MUL_WEIGHT = EPI == kEpiMulWeight;
   constexpr bool GATED = EPI == kEpiGatedSilu;
@@ -317,7 +323,7 @@ static int launch_wide_epilogue(MoeGemmArgs g, int64_t out_cols, int epilogue, h
   }
 }
 
-// Entry used by sarathi_moe_grouped_gemm for row-major weights at 64- and 256-slot blocks.  `g`
+// Entry used by sarathi_moe_grouped_gemm for row-major weights at 64-, 128- and 256-slot blocks.  `g`
 // is complete except for n_blocks, which depends on the epilogue and the column-block width.
 int launch_moe_gemm_wide(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, int dtype,
                          hipStream_t st) {
@@ -334,6 +340,8 @@ int launch_moe_gemm_wide(MoeGemmArgs g, int64_t out_cols, int block_m, int epilo
   if (block_m == 256)                                                                             \
     return narrow ? launch_wide_epilogue<DT, 128, 256>(g, out_cols, epilogue, st)                 \
                   : launch_wide_epilogue<DT, 256, 256>(g, out_cols, epilogue, st);                \
+  if (block_m == 128)                                                                             \
+    return launch_wide_epilogue<DT, 256, 128>(g, out_cols, epilogue, st);                         \
   return narrow ? launch_wide_epilogue<DT, 128, 64>(g, out_cols, epilogue, st)                    \
                 : launch_wide_epilogue<DT, 256, 64>(g, out_cols, epilogue, st);
   if (dtype == kBF16) { SK_PICK(kBF16) } else { SK_PICK(kF16) }
