@@ -52,6 +52,7 @@ def _close(got, want, what):
     (2100, 4, 2, 128, 256, 64, True),    # 36 blocks of 128
     (1500, 4, 2, 256, 4100, 128, True),  # 16 slot blocks x 17 column blocks: the 256-wide tiles of
                                          # the four-wave kernel (smaller launches take 128-wide ones)
+    (1200, 8, 2, 64, 6148, 64, False),   # 46 blocks of 64 x 25 column blocks: 256-wide tiles at 64 slots
 ])
 def test_grouped_gemm_matches_formulation(ops, dev, dtype, T, E, k, BM, N, K, mul):
     _, w, ids, s, e, p = _route(T, E, k, BM, T + N)
