@@ -245,3 +245,51 @@ def test_kv_append_routing_and_expert_gemm_under_hip_graph_capture(ops, dev):
         for a, b in zip(outs, want):
             assert torch.equal(a, b), "replay %d differs from the eager run" % it
         _ = (x.float().sum() + gating.sum()).item()
+
+
+def test_mixtral_expert_gemms_full_size(ops, dev):
+    """The grouped expert GEMMs at the Mixtral-8x7B layer's real shape (4096 tokens, 8 experts,
+    top-2, hidden 4096, intermediate 14336), where a CPU formulation of the whole product would take
+    minutes.  Size-independent checks: (1) the two weight layouts run two different kernels (four
+    waves with both operands through LDS; eight waves with the weights straight into registers)
+    that form every output from the same products in the same order, so their results must agree
+    bit for bit; (2) doubling the activations doubles every output exactly (power-of-two scaling
+    commutes with every rounding as long as nothing overflows); (3) a random sample of outputs
+    against float64 dot products of the gathered rows; (4) the gated epilogue against the separate
+    activation kernel."""
+    from sarathi_amd import layers
+    T, E, k, H, I = 4096, 8, 2, 4096, 14336
+    bf = torch.bfloat16
+    torch.manual_seed(11)
+    x = torch.randn((T, H), device=dev, dtype=torch.float32).to(bf)
+    w1 = (torch.randn((E, 2 * I, H), device=dev, dtype=torch.float32) * H ** -0.5).to(bf)
+    gating = torch.randn((T, E), device=dev, dtype=torch.float32)
+    tw, ti = layers.fused_topk(x, gating, k, True)
+    config = dict(layers.try_get_optimal_moe_config((E, 2 * I, H), (E, H, I), k, T, packed=False))
+    bm = config["BLOCK_SIZE_M"]
+    s, e, p = layers.moe_align_block_size(ti, bm, E)
+
+    def run(a, b, packed, gated):
+        c = torch.full((T * k, I if gated else 2 * I), 3.0, device=dev, dtype=bf)
+        ops.moe_ops.moe_grouped_gemm(a, b, c, tw, s, e, p, T * k, bm, k, False, packed, 2 * I, gated)
+        return c
+
+    plain = run(x, w1, False, False)
+    packed_w1 = layers.pack_expert_weights(w1).data
+    assert torch.equal(run(x, packed_w1, True, False), plain)            # (1)
+    assert torch.equal(run(x * 2, w1, False, False), plain * 2)          # (2)
+    # (3) 256 sampled outputs
+    g = gen(12)
+    slots = torch.randint(0, T * k, (256,), generator=g)
+    cols = torch.randint(0, 2 * I, (256,), generator=g)
+    xs = x[(slots // k).to(dev)].double().cpu()
+    experts = ti.flatten()[slots.to(dev)].long()
+    ws = w1[experts, cols.to(dev)].double().cpu()
+    want = (xs * ws).sum(-1)
+    got = plain[slots.to(dev), cols.to(dev)].double().cpu()
+    assert bool(((got - want).abs() <= 1e-2 * want.abs() + 1e-2).all()), (got - want).abs().max()
+    # (4)
+    act = torch.empty((T * k, I), device=dev, dtype=bf)
+    ops.activation_ops.silu_and_mul(act, plain)
+    assert torch.equal(run(x, w1, False, True), act)
+    assert torch.equal(run(x, packed_w1, True, True), act)
