@@ -16,7 +16,9 @@ ops), µs per call, GB/s and fraction of the 8 TB/s HBM peak, cold and warm (sam
 call).  `roofline` describes the dominant kernel of the step, silu_and_mul: its algorithmic bytes
 divided by its average launch duration over --steps back-to-back launches on cold buffers between
 two HIP events on the launch stream.  `cpu_baseline` is the PyTorch CPU formulation of the same
-step on this machine's host cores.
+step on this machine's host cores.  `moe_layer` times the MoE layer that the routing ops feed
+(`fused_moe` forward with the grouped expert GEMMs, Mixtral-8x7B shape, row-major weights) at
+three batch sizes; it is reported beside the headline, not in it.
 
 --calibrate-copy additionally runs a plain device-to-device copy of a known size (256 MiB,
 torch's copy kernel) so that a `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` run of this script can
@@ -382,6 +384,46 @@ def main():
                           ["fused_add_rms_norm", "rms_norm", "rotary_embedding", "silu_and_mul"]),
     }
 
+    # ---- the MoE layer either side of the routing ops: fused_moe forward (routing, slot sort, both
+    # grouped expert GEMMs with the activation in the first one's epilogue, top-k sum) at the
+    # Mixtral-8x7B layer shape with the reference's row-major [E, N, K] weights.  MFMA-bound at
+    # large batches, weight-streaming-bound at decode sizes; not part of `value`.
+    def measure_moe_layer():
+        from sarathi_amd import layers
+        E, k, H, I = 8, 2, 4096, 14336
+        bf = torch.bfloat16
+        w1 = (torch.randn((E, 2 * I, H), device=dev, dtype=torch.float32) * H ** -0.5).to(bf)
+        w2 = (torch.randn((E, H, I), device=dev, dtype=torch.float32) * I ** -0.5).to(bf)
+        rows = {}
+        for Tn in (16, 1024, 4096):
+            x = torch.randn((Tn, H), device=dev, dtype=torch.float32).to(bf)
+            logits = torch.randn((Tn, E), device=dev, dtype=torch.float32)
+            fn = lambda: layers.fused_moe(x, w1, w2, logits, k, True)  # noqa: E731
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            reps = 20
+            a.record()
+            for _ in range(reps):
+                fn()
+            b.record()
+            torch.cuda.synchronize()
+            ms = a.elapsed_time(b) / reps
+            flop = 2.0 * Tn * k * 3 * I * H
+            rows["%d tokens" % Tn] = {
+                "ms": round(ms, 4), "TFLOPs": round(flop / ms * 1e-9, 1),
+                "frac_of_mfma_peak": round(flop / ms * 1e-9 / 2500.0, 4),
+                "weight_stream_TBps": round((E * 3 * I * H * 2) / ms * 1e-9, 2)}
+        del w1, w2
+        torch.cuda.empty_cache()
+        return {"shape": "Mixtral-8x7B MoE layer: 8 experts, top-2, hidden 4096, intermediate 14336, "
+                         "bf16, row-major weights, back-to-back launches (weights warm in L2/MALL "
+                         "as far as they fit)",
+                "peak": "2500 TFLOP/s dense bf16 MFMA; 8 TB/s HBM", "fused_moe_forward": rows}
+
+    moe_layer = measure_moe_layer()
+
     silu_us = per_op["silu_and_mul"]["cold"]["us"]
     silu_gbs = BYTES["silu_and_mul"] / silu_us * 1e-3
     roofline = {
@@ -482,6 +524,7 @@ def main():
         "cpu_baseline": cpu,
         "per_op": per_op,
         "other_configs": other_configs,
+        "moe_layer": moe_layer,
         "plain_copy_same_bytes_cold": copy_ref,
     }
     print(json.dumps(out))
