@@ -134,9 +134,17 @@ def try_get_optimal_moe_config(w1_shape: Tuple[int, ...], w2_shape: Tuple[int, .
                                override_config: Optional[Dict[str, Any]] = None,
                                packed: bool = True) -> Dict[str, Any]:
     """override_config, else the tuned entry closest to M, else the default rule
-    (reference: fused_moe.py:321-343)."""
+    (reference: fused_moe.py:321-343).  An override written for the reference's Triton kernel may
+    name a slot-block size this library's kernels do not have (the reference's default for tiny
+    batches is 16): it is raised to the next size that exists, the other keys pass through."""
     if override_config:
-        return override_config
+        block_m = int(override_config["BLOCK_SIZE_M"])
+        if block_m in _BLOCK_SIZES:
+            return override_config
+        config = dict(override_config)
+        config["BLOCK_SIZE_M"] = min((b for b in _BLOCK_SIZES if b >= block_m),
+                                     default=max(_BLOCK_SIZES))
+        return config
     E, _, N = w2_shape
     configs = get_moe_configs(E, N, dtype, packed)
     if configs:

@@ -132,3 +132,19 @@ def test_pack_expert_weights_layout_and_inplace():
     # rows beyond N are zero padding
     odd = fm.pack_expert_weights(torch.ones((1, 40, 16)))
     assert odd.data.shape == (1, 2, 1, 2, 32, 8) and odd.data[0, 1, 0, :, 8:, :].abs().sum() == 0
+
+
+def test_override_config_block_size_is_raised_to_one_that_exists():
+    """A config tuned for the reference's Triton kernel (fused_moe.py:297-318 defaults to
+    BLOCK_SIZE_M = 16 for tiny batches) must not be rejected: the block size is raised to the next
+    one the kernels have, everything else passes through; supported sizes are returned as given."""
+    import importlib
+    fm = importlib.import_module("sarathi_amd.layers.fused_moe")
+    ref = {"BLOCK_SIZE_M": 16, "BLOCK_SIZE_N": 32, "BLOCK_SIZE_K": 64, "GROUP_SIZE_M": 1}
+    got = fm.try_get_optimal_moe_config((8, 28672, 4096), (8, 4096, 14336), 2, 4, override_config=ref)
+    assert got["BLOCK_SIZE_M"] == 32 and got["BLOCK_SIZE_N"] == 32 and ref["BLOCK_SIZE_M"] == 16
+    for bm in (32, 64, 128, 256):
+        cfg = {"BLOCK_SIZE_M": bm}
+        assert fm.try_get_optimal_moe_config((8, 8, 64), (8, 64, 4), 2, 4, override_config=cfg) is cfg
+    big = fm.try_get_optimal_moe_config((8, 8, 64), (8, 64, 4), 2, 4, override_config={"BLOCK_SIZE_M": 512})
+    assert big["BLOCK_SIZE_M"] == 256
