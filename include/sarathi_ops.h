@@ -235,6 +235,18 @@ int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c, const float*
                              int top_k, int epilogue, int b_layout, int dtype, void* stream);
 
 /*
+ * Replaces the torch.sum(intermediate_cache3, dim=1, out=...) that ends fused_experts
+ * (sarathi/model_executor/layers/fused_moe/fused_moe.py:539-543): out[t, :] = sum over j of
+ * input[t, j, :] for the top_k expert outputs of token t, fp32 accumulation in ascending j, one
+ * rounding to the tensor dtype.  input row (t, j) starts at t * in_token_stride + j * in_k_stride
+ * elements, out row t at t * out_row_stride; rows are `hidden` contiguous elements.
+ * dtype: SARATHI_DTYPE_F32 / F16 / BF16.
+ */
+int sarathi_moe_sum(void* out, const void* input, int64_t num_tokens, int64_t top_k,
+                    int64_t hidden, int64_t in_token_stride, int64_t in_k_stride,
+                    int64_t out_row_stride, int dtype, void* stream);
+
+/*
  * Paged KV cache (NHD page layout: entry e of page p holds [num_kv_heads, head_size] elements and
  * starts page_stride*p + entry_stride*e elements after k_cache, resp. v_cache; the reference's
  * cache tensor [num_pages, 2, page_size, num_kv_heads, head_size],

@@ -22,7 +22,7 @@ LIB_DIR = os.path.join(PKG, "lib")
 OBJ_DIR = os.path.join(HERE, "build", "obj")
 
 HIP_SOURCES = ["rms_norm.hip", "gated_act.hip", "rope.hip", "moe_topk.hip", "moe_align.hip",
-               "moe_gemm.hip", "moe_gemm_wide.hip", "kv_cache.hip",
+               "moe_gemm.hip", "moe_gemm_wide.hip", "moe_sum.hip", "kv_cache.hip",
                "moe_fused_routing.hip"]
 CXX_SOURCES = ["abi_misc.cpp"]
 

@@ -578,6 +578,25 @@ void fused_topk_align(torch::Tensor& topk_weights, torch::Tensor& topk_indices,
            op);
 }
 
+// torch.sum(input, dim=1, out=out) of fused_moe.py:539-543: input [tokens, top_k, hidden]
+void moe_sum(torch::Tensor& input, torch::Tensor& out) {
+  const char* op = "moe_sum";
+  check_gpu(input, input, op, "input");
+  check_gpu(out, input, op, "out");
+  TORCH_CHECK(input.dim() == 3 && out.dim() == 2, op, ": input [tokens, top_k, hidden], out [tokens, hidden]");
+  TORCH_CHECK(out.size(0) == input.size(0) && out.size(1) == input.size(2), op,
+              ": out must be [input.size(0), input.size(2)]");
+  TORCH_CHECK(out.scalar_type() == input.scalar_type(), op, ": out and input must share a dtype");
+  TORCH_CHECK(input.size(1) >= 1, op, ": top_k must be at least 1");
+  TORCH_CHECK((input.stride(2) == 1 || input.size(2) <= 1) && (out.stride(1) == 1 || out.size(1) <= 1),
+              op, ": rows must be contiguous");
+  LaunchScope scope(input);
+  raise_on(sarathi_moe_sum(out.data_ptr(), input.data_ptr(), input.size(0), input.size(1),
+                           input.size(2), input.stride(0), input.stride(1), out.stride(0),
+                           dtype_code(input, op), scope.stream),
+           op);
+}
+
 // A [tokens, K], B [E, N, K], C [tokens, topk, N] (or any tensor whose rows of N elements are
 // addressed by slot = token * topk + j), as invoke_fused_moe_kernel passes them.  With
 // b_packed, B is the re-tiled weight tensor [E, ceil(N/32), K/16, 2, 32, 8] and `n` its logical
@@ -654,6 +673,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("fused_add_rms_norm", &fused_add_rms_norm,
         "residual += input; input = rms_norm(residual) * weight (both in place)");
   // activation_ops
+  m.def("moe_sum", &moe_sum, "out[t] = sum over the top_k rows of input[t]");
   m.def("silu_and_mul", &silu_and_mul, "out = silu(input[:, :d]) * input[:, d:]");
   m.def("gelu_new", &gelu_new, "GPT-2 tanh GELU");
   m.def("gelu_fast", &gelu_fast, "approximate tanh GELU");

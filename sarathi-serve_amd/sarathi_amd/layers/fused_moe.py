@@ -231,7 +231,7 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
             activation_ops.silu_and_mul(c2, c1.view(-1, N))
         invoke_fused_moe_kernel(c2, w2, c3, None, None, cur_w, cur_ids, sorted_ids, expert_ids,
                                 post_padded, True, 1, config)
-        torch.sum(c3, dim=1, out=out[begin:end])
+        moe_ops.moe_sum(c3, out[begin:end])   # the reference's torch.sum(c3, dim=1, out=...)
     return out
 
 

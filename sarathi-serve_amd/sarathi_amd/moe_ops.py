@@ -22,5 +22,9 @@ fused_topk_align = _C.fused_topk_align
 # the group-limited routing the reference writes with tensor ops (fused_moe.py:377-408)
 grouped_topk = _C.grouped_topk
 
-__all__ = ["topk_softmax", "moe_align_block_size", "topk_softmax_renorm",
+# moe_sum(input[tokens, top_k, hidden], out[tokens, hidden]): the torch.sum over the top-k expert
+# outputs that ends fused_experts (fused_moe.py:539-543)
+moe_sum = _C.moe_sum
+
+__all__ = ["moe_sum", "topk_softmax", "moe_align_block_size", "topk_softmax_renorm",
            "moe_align_block_size_filled", "moe_grouped_gemm", "fused_topk_align", "grouped_topk"]
