@@ -162,6 +162,27 @@ def test_gpu_activations_any_shape(ops, dev, T, d, dt, seed):
 
 @pytest.mark.gpu
 @GPU
+@given(T=st.integers(0, 40), k=st.integers(1, 8), H=st.integers(1, 700), dt=st.sampled_from(DTYPES),
+       pad_k=st.integers(0, 2), pad_h=st.sampled_from([0, 8, 24]), seed=st.integers(0, 10 ** 6))
+def test_gpu_moe_sum_any_shape(ops, dev, T, k, H, dt, pad_k, pad_h, seed):
+    """Any shape, dtype and input strides against the library sum: two addends bit for bit, more
+    within one ulp of the dtype (the fp32 order of additions may differ)."""
+    g = gen(seed)
+    big = randn((T, k + pad_k, H + pad_h), g, dt, std=1.5)
+    x = big[:, :k, :H]
+    want = torch.sum(x, dim=1)
+    got = torch.full((T, H), 5.0, dtype=dt, device=dev)
+    ops.moe_ops.moe_sum(big.to(dev)[:, :k, :H], got)
+    if k <= 2:
+        assert torch.equal(got.cpu(), want)
+    elif dt == torch.float32:
+        torch.testing.assert_close(got.cpu(), want, atol=4e-6, rtol=4e-6)
+    else:
+        assert_close_dtype(got, want, max_ulps=1)
+
+
+@pytest.mark.gpu
+@GPU
 @given(E=st.integers(1, 300), B=st.sampled_from([1, 4, 16, 64, 128]), n=st.integers(0, 3000),
        idt=st.sampled_from([torch.uint8, torch.int16, torch.int32, torch.int64]),
        seed=st.integers(0, 10 ** 6), skew=st.booleans(), fill=st.booleans())
