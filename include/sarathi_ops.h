@@ -207,7 +207,10 @@ int sarathi_fused_topk_align(float* topk_weights, int32_t* topk_indices,
  *       [num_valid_tokens, N/2] = silu_and_mul of the [.., N] product, with the rounding points
  *       of the unfused sequence GEMM -> silu_and_mul (fused_moe.py:499-520), so results are
  *       bit-identical to it while the [.., N] intermediate never reaches memory.  N/2 must be a
- *       multiple of 4 (of 32 with packed weights).  A [tokens, K] with rows a_row_stride elements apart, B
+ *       multiple of 4 (of 32 with packed weights).
+ * A [tokens, K] with rows a_row_stride elements apart; A MUST hold at least
+ * ceil(num_valid_tokens / top_k) rows (the kernel derives the extent of its reads from that
+ * figure, not from the allocation) and top_k must be positive.  B
  * [E, N, K] K-contiguous with experts b_expert_stride elements apart, C
  * [num_valid_tokens, N] with rows c_row_stride apart (num_valid_tokens =
  * tokens * topk; slots holding a larger id are padding and skipped).

@@ -5,7 +5,8 @@
 // bound, so a kernel boundary (drain, launch, ramp) is a large part of their cost.  Here
 // workgroups of 16 waves compute the top-k of 16 row blocks each, exactly as the stand-alone
 // kernel does, except that the expert ids are stored as device-scope atomics (written through to
-// where every compute unit reads coherently); once its stores have completed every workgroup
+// where every compute unit reads coherently); once every wave has waited for the
+// acknowledgement of its stores (s_waitcnt vmcnt(0)) and met the others at a barrier, the workgroup
 // bumps a counter in global memory, and the workgroup that sees the last count runs the
 // single-workgroup sort, reading the ids of all workgroups with device-scope loads.  (A full
 // device-scope fence on either side also works but costs several microseconds of cache
@@ -41,7 +42,12 @@ __global__ __launch_bounds__(64 * kFusedWaves) void fused_topk_align_kernel(
   if (block < row_blocks)  // uniform over the wave
     topk_rows_pow2<E, true>(block, weights, indices, source, gating, num_tokens, k, renormalize);
 
-  // the barrier's workgroup-scope release makes every wave wait for its outstanding stores
+  // Publication: the ids above are write-through (device-scope) stores, and their
+  // acknowledgement, which vmcnt counts, comes back once they are where every compute unit reads
+  // coherently.  Every wave waits for its own stores here; the barrier that follows then tells
+  // thread 0 that all ids of this workgroup are visible before it bumps the counter.  (The
+  // barrier alone does not: its workgroup-scope fence does not wait for global stores.)
+  wait_vmcnt<0>();
   __syncthreads();
   if (threadIdx.x == 0) {
     const uint32_t prev = atomicAdd(counter, 1u);

@@ -49,9 +49,6 @@ SK_DEV void dma_load16_to_lds(rsrc_t r, u32x4* lds_base, uint32_t byte_off) {
       r, (__attribute__((address_space(3))) void*)lds_base, 16, byte_off, 0, 0, 0);
 }
 
-// Waits until at most N vector-memory operations of this wave are outstanding.
-template <int N> SK_DEV void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
-
 struct MoeGemmArgs {
   const void* a;            // [tokens, K]
   const void* b;            // [E, N, K]

@@ -616,6 +616,10 @@ void moe_grouped_gemm(torch::Tensor& a, torch::Tensor& b, torch::Tensor& c,
   check_gpu(num_tokens_post_padded, a, op, "num_tokens_post_padded");
   TORCH_CHECK(a.dim() == 2 && a.stride(1) == 1, op, ": A must be [tokens, K] with contiguous rows");
   const int64_t k = a.size(1);
+  // the kernel gathers row slot / top_k of A for every slot below num_valid_tokens
+  TORCH_CHECK(top_k > 0 && num_valid_tokens >= 0 && a.size(0) * top_k >= num_valid_tokens, op,
+              ": A has ", a.size(0), " rows but num_valid_tokens = ", num_valid_tokens,
+              " with top_k = ", top_k, " needs ceil(num_valid_tokens / top_k)");
   int64_t expert_stride;
   if (b_packed) {
     TORCH_CHECK(b.dim() == 6 && b.is_contiguous() && b.size(3) == 2 && b.size(4) == 32 &&

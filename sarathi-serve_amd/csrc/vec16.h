@@ -157,13 +157,20 @@ template <int DT> SK_DEV void store_elem(void* base, int64_t i, float v) {
   else reinterpret_cast<_Float16*>(base)[i] = (_Float16)v;
 }
 
-// ---- workgroup barrier for LDS exchanges ---------------------------------------
+// ---- waits and the workgroup barrier for LDS exchanges ---------------------------
 
-// Orders LDS traffic only.  __syncthreads() also waits for every outstanding global access of
-// the wave (its release fence drains vmcnt, which on gfx9 counts loads and stores alike), i.e.
-// for prefetches and streaming stores that are meant to stay in flight across the barrier;
-// here a wave waits for its own LDS operations and then meets the others.  Use it only where
-// the data exchanged through the barrier lives in LDS.
+// Waits until at most N of this wave's vector-memory operations (loads and stores alike on
+// gfx9) are outstanding.
+template <int N> SK_DEV void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
+// Orders LDS traffic only: a wave waits for its own LDS operations and then meets the others.
+// Global loads and stores issued before it stay in flight across it (prefetches, streaming
+// stores).  __syncthreads() promises no more than that for global memory on this target: its
+// fences are workgroup scope, and when all waves of a workgroup share a compute unit the
+// compiler may satisfy them without a `vmcnt(0)` (it usually waits for fewer operations, or
+// none).  Data that has to be visible outside the workgroup needs an explicit
+// wait_vmcnt<0>() (for write-through stores) or a wider fence.  Use this barrier only where
+// the data exchanged through it lives in LDS.
 SK_DEV void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
