@@ -42,6 +42,7 @@ extern "C" {
 #define SARATHI_ERR_INVALID_ARG (-1) /* null pointer, negative size, bad stride */
 #define SARATHI_ERR_UNSUPPORTED (-2) /* unknown dtype code or shape outside limits */
 #define SARATHI_ERR_LAUNCH (-3)      /* the HIP runtime rejected the launch */
+#define SARATHI_ERR_SCRATCH_LIMIT (-4) /* input needs more than the fixed scratch of a *_static entry */
 
 /* Largest num_experts accepted by the two MoE routing entry points. */
 #define SARATHI_MOE_MAX_EXPERTS 1024
@@ -160,6 +161,31 @@ int sarathi_moe_align_block_size(const void* topk_ids, int id_dtype, int64_t num
  * (csrc/moe_topk_softmax_kernels.cu:486-492).
  */
 int64_t sarathi_moe_align_workspace_bytes(int64_t numel, int num_experts);
+
+/*
+ * sarathi_moe_align_block_size for callers that cannot allocate device memory or bring a
+ * workspace (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * It has no counterpart in the reference.  Same arguments, results and error codes as
+ * sarathi_moe_align_block_size without `workspace`; the scratch of the three-launch path for
+ * inputs above 16 K ids is a fixed array of SARATHI_MOE_ALIGN_STATIC_SCRATCH_BYTES that lives in
+ * the library's device image (every GPU the library runs on holds it until the process ends).
+ * The call allocates and frees nothing.  Inputs for which
+ * sarathi_moe_align_workspace_bytes(numel, num_experts) exceeds that size are refused with
+ * SARATHI_ERR_SCRATCH_LIMIT (with 255 experts or fewer every numel fits; 1024 experts fit up to
+ * 129 024 ids) and nothing is launched.  All calls on one GPU share the one array: calls that
+ * overlap on the same GPU (different streams, or different host threads without ordering between
+ * their launches) race on it; calls on one stream are safe.  The array's contents between calls
+ * are irrelevant: every word a call reads it has written before.  This is the one entry point of
+ * the library that keeps state (the per-device address of the array, looked up on the first call on
+ * each device).
+ */
+#define SARATHI_MOE_ALIGN_STATIC_SCRATCH_BYTES (1 << 20)
+int sarathi_moe_align_block_size_static(const void* topk_ids, int id_dtype, int64_t numel,
+                                        int num_experts, int block_size,
+                                        int32_t* sorted_token_ids, int64_t sorted_len,
+                                        int32_t* expert_ids, int64_t expert_ids_len,
+                                        int32_t* num_tokens_post_pad, int fill_pad,
+                                        void* stream);
 
 /*
  * Replaces grouped_topk(hidden_states, gating_output, topk, renormalize, num_expert_group,

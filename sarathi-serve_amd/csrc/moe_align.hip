@@ -28,6 +28,8 @@
 //
 // Each LDS counter has a single writer wave, there is no global scratch and no
 // inter-workgroup traffic, so the result is deterministic and bit-exact.
+#include <atomic>
+
 #include "moe_align_body.h"
 #include "launch.h"
 
@@ -260,6 +262,40 @@ static int launch_align(const void* ids, int64_t numel, int E, int B, int32_t* s
   return launch_status();
 }
 
+// ---------------------------------------------------------------------------
+// Scratch of the entry point that allocates nothing.  `scratch` is a host-side
+// stand-in for the device array, not a device address: host code goes through
+// the address hipGetSymbolAddress returns for the current device, fetched once
+// per device (every GPU holds its own copy of the array at its own address).
+// ---------------------------------------------------------------------------
+constexpr int64_t kStaticScratchInts = SARATHI_MOE_ALIGN_STATIC_SCRATCH_BYTES / 4;
+static __device__ __align__(256) int32_t scratch[kStaticScratchInts];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<int32_t*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device, or null with *status set.
+static int32_t* static_scratch(int* status) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    *status = SARATHI_ERR_LAUNCH;
+    return nullptr;
+  }
+  int32_t* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    void* sym = nullptr;
+    if (hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)) != hipSuccess || sym == nullptr) {
+      (void)hipGetLastError();
+      *status = SARATHI_ERR_LAUNCH;
+      return nullptr;
+    }
+    p = reinterpret_cast<int32_t*>(sym);
+    // two threads racing here fetch the same address for the same device
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  return p;
+}
+
 }  // namespace sarathi_hip
 
 extern "C" int64_t sarathi_moe_align_workspace_bytes(int64_t numel, int num_experts) {
@@ -304,4 +340,28 @@ extern "C" int sarathi_moe_align_block_size(const void* topk_ids, int id_dtype, 
     default: return SARATHI_ERR_UNSUPPORTED;
   }
 #undef SK_ALIGN
+}
+
+extern "C" int sarathi_moe_align_block_size_static(const void* topk_ids, int id_dtype,
+                                                   int64_t numel, int num_experts,
+                                                   int block_size, int32_t* sorted_token_ids,
+                                                   int64_t sorted_len, int32_t* expert_ids,
+                                                   int64_t expert_ids_len,
+                                                   int32_t* num_tokens_post_pad, int fill_pad,
+                                                   void* stream) {
+  using namespace sarathi_hip;
+  // 0 for inputs that take the single-workgroup path, which uses no global scratch
+  const int64_t need = sarathi_moe_align_workspace_bytes(numel, num_experts);
+  if (need > SARATHI_MOE_ALIGN_STATIC_SCRATCH_BYTES) return SARATHI_ERR_SCRATCH_LIMIT;
+  int32_t* ws = nullptr;
+  if (need > 0) {
+    int status = SARATHI_OK;
+    ws = static_scratch(&status);
+    if (ws == nullptr) return status;
+  }
+  // every word of the scratch that the scan and scatter kernels read is written by the count
+  // and scan kernels of the same call, so nothing has to be cleared between calls
+  return sarathi_moe_align_block_size(topk_ids, id_dtype, numel, num_experts, block_size,
+                                      sorted_token_ids, sorted_len, expert_ids, expert_ids_len,
+                                      num_tokens_post_pad, fill_pad, ws, need, stream);
 }

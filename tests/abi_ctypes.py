@@ -25,6 +25,7 @@ _SIGNATURES = {
     "sarathi_rotary_embedding": [vp, vp, vp, vp, i64, ci, ci, ci, ci, i64, i64, ci, ci, vp],
     "sarathi_topk_softmax": [vp, vp, vp, vp, i64, ci, ci, ci, vp],
     "sarathi_moe_align_block_size": [vp, ci, i64, ci, ci, vp, i64, vp, i64, vp, ci, vp, i64, vp],
+    "sarathi_moe_align_block_size_static": [vp, ci, i64, ci, ci, vp, i64, vp, i64, vp, ci, vp],
     "sarathi_moe_sum": [vp, vp, i64, i64, i64, i64, i64, i64, ci, vp],
 }
 

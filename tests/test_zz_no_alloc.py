@@ -1,0 +1,90 @@
+"""sarathi_moe_align_block_size_static, the entry point that allocates nothing (its scratch is a
+fixed array inside the library's device image), called through the C ABI and compared bit for bit
+with sarathi_moe_align_block_size given a caller-provided workspace, and with the CPU oracle.
+Two calls in a row share the array, the second with a smaller input.  Collected last on purpose.
+"""
+import pytest
+import torch
+
+import abi_ctypes as abi
+from oracle import c_oracle
+
+pytestmark = pytest.mark.gpu
+
+SCRATCH_LIMIT = -4
+
+
+def _run(lib, fn_static, ids_dev, E, B, fill_pad):
+    numel = ids_dev.numel()
+    s, e, p = abi.align_buffers(numel, E, B, ids_dev.device, fill=numel if not fill_pad else -3)
+    args = [abi.ptr(ids_dev), abi.ID_DT[ids_dev.dtype], numel, E, B, abi.ptr(s), s.numel(),
+            abi.ptr(e), e.numel(), abi.ptr(p), int(fill_pad)]
+    if fn_static:
+        rc = lib.sarathi_moe_align_block_size_static(*args, abi.stream())
+        ws = None
+    else:
+        need = lib.sarathi_moe_align_workspace_bytes(numel, E)
+        ws = torch.empty((max(need, 4),), dtype=torch.uint8, device=ids_dev.device)
+        rc = lib.sarathi_moe_align_block_size(*args, abi.ptr(ws), need, abi.stream())
+    abi.check(lib, rc)
+    torch.cuda.synchronize()
+    return s.cpu(), e.cpu(), p.cpu()
+
+
+def _oracle(ids, E, B):
+    numel = ids.numel()
+    s, e, p = (t.cpu() for t in abi.align_buffers(numel, E, B, "cpu"))
+    c_oracle.moe_align_block_size(ids, E, B, s, e, p)
+    return s, e, p
+
+
+def _same(got, want, B):
+    assert torch.equal(got[2], want[2])
+    assert torch.equal(got[0], want[0])
+    nblk = int(want[2].item()) // B
+    assert torch.equal(got[1][:nblk], want[1][:nblk])
+    assert bool((got[1][nblk:] == -7).all())
+
+
+def test_static_scratch_entry_matches_workspace_entry_twice(dev):
+    lib = abi.load()
+    g = torch.Generator().manual_seed(41)
+    # both sizes take the three-launch path (above 16 384 ids), i.e. both use the scratch; the
+    # second call is smaller, so stale words of the first call's table lie beyond what it writes
+    cases = [(200_000, 64, 32, torch.int32), (40_000, 8, 64, torch.int64), (17_000, 5, 16, torch.int16)]
+    for numel, E, B, dt in cases:
+        ids = torch.randint(0, E, (numel,), generator=g, dtype=torch.int32).to(dt)
+        assert lib.sarathi_moe_align_workspace_bytes(numel, E) > 0
+        ids_dev = ids.to(dev)
+        for fill_pad in (0, 1):
+            got = _run(lib, True, ids_dev, E, B, fill_pad)
+            want = _run(lib, False, ids_dev, E, B, fill_pad)
+            _same(got, want, B)
+            _same(got, _oracle(ids, E, B), B)
+
+
+def test_static_scratch_entry_small_inputs_and_limit(dev):
+    lib = abi.load()
+    g = torch.Generator().manual_seed(42)
+    # at or below 16 384 ids the single-workgroup path runs: no scratch at all
+    for numel, E, B in [(8192, 8, 64), (1, 8, 4), (0, 8, 4)]:
+        ids = torch.randint(0, E, (numel,), generator=g, dtype=torch.int32)
+        got = _run(lib, True, ids.to(dev), E, B, 1)
+        _same(got, _oracle(ids, E, B), B)
+    # 1024 experts and 252 * 512 ids is the largest table that fits; one chunk group more does not
+    E, B = 1024, 4
+    for numel, ok in [(129_024, True), (129_025, False)]:
+        ids = torch.randint(0, E, (numel,), generator=g, dtype=torch.int32)
+        ids_dev = ids.to(dev)
+        s, e, p = abi.align_buffers(numel, E, B, dev, fill=-3)
+        rc = lib.sarathi_moe_align_block_size_static(
+            abi.ptr(ids_dev), abi.ID_DT[ids.dtype], numel, E, B, abi.ptr(s), s.numel(), abi.ptr(e),
+            e.numel(), abi.ptr(p), 1, abi.stream())
+        torch.cuda.synchronize()
+        if ok:
+            abi.check(lib, rc)
+            _same((s.cpu(), e.cpu(), p.cpu()), _oracle(ids, E, B), B)
+        else:
+            assert rc == SCRATCH_LIMIT
+            assert b"scratch" in lib.sarathi_ops_strerror(rc)
+            assert p.item() == -7 and bool((s == -3).all())  # nothing was launched
