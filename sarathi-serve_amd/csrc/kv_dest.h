@@ -36,21 +36,40 @@ struct KvDest {
   int32_t page_size;
 };
 
-// Byte offset of token `tok`'s entry from k_cache / v_cache.  `tok` is uniform over the wave, so
-// the four dependent loads are scalar loads.
-SK_DEV int64_t kv_entry_offset(const KvDest& d, int64_t tok) {
+// Byte offset of token `tok`'s entry from k_cache / v_cache, in two steps so that a kernel can
+// put other work between them: kv_entry_key() issues the scalar loads that depend on nothing but
+// the token index, kv_entry_resolve() the dependent page-table lookups.  `tok` is uniform over
+// the wave, so all of these are scalar loads.
+struct KvEntryKey {
+  int32_t a;  // slot (with a slot mapping) or request index
+  int32_t b;  // position of the token inside its request's kv sequence (unused with a mapping)
+};
+SK_DEV KvEntryKey kv_entry_key(const KvDest& d, int64_t tok) {
+  KvEntryKey k;
   if (d.slot_mapping != nullptr) {
-    const uint32_t slot = (uint32_t)d.slot_mapping[tok];
+    k.a = d.slot_mapping[tok];
+    k.b = 0;
+  } else {
+    k.a = d.batch_indices[tok];
+    k.b = d.positions[tok];
+  }
+  return k;
+}
+SK_DEV int64_t kv_entry_resolve(const KvDest& d, KvEntryKey k) {
+  if (d.slot_mapping != nullptr) {
+    const uint32_t slot = (uint32_t)k.a;
     const uint32_t page = slot / (uint32_t)d.page_size;
     const uint32_t entry = slot - page * (uint32_t)d.page_size;
     return (int64_t)page * d.page_stride_bytes + (int64_t)entry * d.entry_stride_bytes;
   }
-  const int32_t b = d.batch_indices[tok];
-  const uint32_t pos = (uint32_t)d.positions[tok];
+  const uint32_t pos = (uint32_t)k.b;
   const uint32_t pg = pos / (uint32_t)d.page_size;
   const uint32_t entry = pos - pg * (uint32_t)d.page_size;
-  const int64_t page = d.kv_indices[(int64_t)d.kv_indptr[b] + pg];
+  const int64_t page = d.kv_indices[(int64_t)d.kv_indptr[k.a] + pg];
   return page * d.page_stride_bytes + (int64_t)entry * d.entry_stride_bytes;
+}
+SK_DEV int64_t kv_entry_offset(const KvDest& d, int64_t tok) {
+  return kv_entry_resolve(d, kv_entry_key(d, tok));
 }
 
 }  // namespace sarathi_hip

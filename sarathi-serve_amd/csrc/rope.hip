@@ -9,17 +9,26 @@
 //          them in registers and writes both vectors back;
 //   GPT-J: x and y interleave, so one 16-byte vector already holds whole
 //          pairs; cos and sin come from two half-width loads.
-// A workgroup is one wave: 64 consecutive slots of one token's q row or of its
-// k row (8 heads of 128 at bf16).  Workgroup ids run over the q segments, then
-// the k segments, then the tokens, so the waves in flight sweep the packed qkv
-// buffer linearly.  The token's q row, k row and cos/sin cache row are scalar
-// buffer resources (the position is a scalar load); lanes past the last head
-// are clipped by the hardware range check, so the kernel has no branches.
-// Elements at or beyond rot_dim inside a head are not touched.
+// 64 consecutive slots of a token's q row or of its k row (8 heads of 128 at
+// bf16) form a segment.  A workgroup is ONE wave that takes up to five
+// consecutive segments of one token's list (q segments, then k segments): at
+// Llama-3-8B's 32 + 8 heads that is the whole token, so its position and its
+// cos/sin row are fetched once, all of its loads are in flight before the first
+// result is needed, and the launch has one workgroup per token.  (Measured on
+// MI355X at 2304 tokens: one wave per segment 9.3 us, one wave per token 8.4 us;
+// a launch of N one-wave workgroups costs about 0.2 ns per workgroup in the
+// dispatcher alone, 3.5 us for the 11520 of the per-segment layout, and
+// multi-wave workgroups lose more to uneven compute-unit load than they gain.)
+// The token's q row, k row and cos/sin cache row are scalar buffer resources
+// (the position is a scalar load issued first and consumed after the data loads
+// have been issued); lanes past the last head are clipped by the hardware range
+// check, so the kernel has no divergent branches.  Elements at or beyond rot_dim
+// inside a head are not touched.
 //
 // Arithmetic is the reference's scalar_t arithmetic: each product and the final
 // sum round to the tensor dtype (csrc/pos_encoding_kernels.cu:32-35):
 //   x' = T( T(x*cos) - T(y*sin) ),  y' = T( T(y*cos) + T(x*sin) ).
+// The two products of a sum are rounded by one packed conversion.
 #include "vec16.h"
 #include "kv_dest.h"
 #include "launch.h"
@@ -44,43 +53,140 @@ struct RopeArgs {
 
 template <int DT> SK_DEV float mul_r(float a, float b) { return rnd<DT>(a * b); }
 
-// Kernel arguments are laid out so that everything the first loads need sits in
-// the first 56 bytes, which the hardware preloads into scalar registers at wave
-// launch: the wave can issue its q/k loads without waiting for an argument fetch,
-// and only then fetches the token's position and, from it, the cos/sin row.
-//   geom  = head_bytes | embed_bytes << 16          (bytes of one head / of rot_dim/2)
-//   heads = num_heads | num_kv_heads << 12 | slot_shift << 24
-// slot_shift = log2(16-byte slots per head); NeoX counts the slots of the x half,
-// GPT-J those of the whole rotated span.
-template <int DT, bool NEOX>
-__global__ __launch_bounds__(64) void rope_seg_kernel(
-    const int64_t* __restrict__ positions, void* query, void* key, const void* __restrict__ cache,
-    int64_t q_stride_bytes, int64_t k_stride_bytes, uint32_t geom, uint32_t heads) {
-  constexpr int N = VecElems<DT>::value;
-  const uint32_t head_bytes = geom & 0xffffu, embed_bytes = geom >> 16;
-  const int num_heads = heads & 0xfffu, num_kv_heads = (heads >> 12) & 0xfffu;
-  const int slot_shift = heads >> 24;
-  const int q_blocks = ((num_heads << slot_shift) + 63) >> 6;
-  const int64_t tok = (int64_t)blockIdx.z * kMaxGridY + blockIdx.y;
-  const bool is_q = (int)blockIdx.x < q_blocks;  // uniform over the wave
-  const int item = ((int)blockIdx.x - (is_q ? 0 : q_blocks)) * 64 + (int)threadIdx.x;
-  const int nheads = is_q ? num_heads : num_kv_heads;
-  const int h = item >> slot_shift;
-  const uint32_t slot = item & ((1 << slot_shift) - 1);
-  char* base = reinterpret_cast<char*>(is_q ? query : key) +
-               tok * (is_q ? q_stride_bytes : k_stride_bytes);
-  const rsrc_t rd = make_rsrc(base, (uint32_t)nheads * head_bytes);
-  const uint32_t xoff = h < nheads ? (uint32_t)h * head_bytes + slot * 16u : kClipped;
+// One rotation with the reference's rounding points.  For 16-bit dtypes the two products of each
+// sum go through ONE packed conversion (v_cvt_pk_*) and come back as floats.
+template <int DT> SK_DEV void rotate(float x, float y, float c, float s, float& ox, float& oy) {
+  if constexpr (DT == kF32) {
+    ox = x * c - y * s;
+    oy = y * c + x * s;
+  } else {
+    const f32x2 a = unpack2<DT>(pack2<DT>(x * c, y * s));
+    const f32x2 b = unpack2<DT>(pack2<DT>(y * c, x * s));
+    ox = a.x - a.y;
+    oy = b.x + b.y;
+  }
+}
 
-  u32x4 xr, yr;
-  xr = buf_load16<kStreamLoad>(rd, xoff);
-  if constexpr (NEOX) yr = buf_load16<kStreamLoad>(rd, xoff + embed_bytes);
-  // keep the position fetch (and everything hanging off it) behind the loads above
+// Rotates the 16-byte slot(s) of one lane: NeoX x vector `xr` and y vector `yr`; GPT-J only `xr`
+// (interleaved pairs).  `cr`/`sr` hold the matching cos / sin values (GPT-J: in the low half).
+template <int DT, bool NEOX>
+SK_DEV void rotate_slot(u32x4& xr, u32x4& yr, const Vec<DT>& c, const Vec<DT>& s) {
+  constexpr int N = VecElems<DT>::value;
+  Vec<DT> x;
+  x.unpack(xr);
+  if constexpr (NEOX) {
+    Vec<DT> y, ox, oy;
+    y.unpack(yr);
+#pragma unroll
+    for (int i = 0; i < N; ++i) rotate<DT>(x.f[i], y.f[i], c.f[i], s.f[i], ox.f[i], oy.f[i]);
+    xr = ox.pack();
+    yr = oy.pack();
+  } else {
+    Vec<DT> o;
+#pragma unroll
+    for (int i = 0; i < N / 2; ++i)
+      rotate<DT>(x.f[2 * i], x.f[2 * i + 1], c.f[i], s.f[i], o.f[2 * i], o.f[2 * i + 1]);
+    xr = o.pack();
+  }
+}
+
+// Store policy of the in-place results.  With a wave per token the rows it rewrites are still in
+// L2 from its own loads; a non-temporal write-back store measured 2 % faster there than the
+// write-through store that wins for out-of-place streams and for the one-segment shape.
+constexpr int kNtStore = 2;
+
+// What a launch works on.  The two row arrays are called A and B: A is whichever of query / key
+// starts lower in memory, and B is reached THROUGH A's per-token buffer resource at byte offset
+// delta0 + token * delta_step (callers pass views of one packed qkv buffer, so this is a small
+// constant), which leaves one resource and no per-segment selects in the kernel.  A token's
+// segment list is A's segments, then B's.
+//   geom  = head_bytes | embed_bytes << 16          (bytes of one head / of rot_dim/2)
+//   heads = heads of A | heads of B << 12 | slot_shift << 24 | (A is the key array) << 31
+// slot_shift = log2(16-byte slots per head), at most 6; NeoX counts the slots of the x half,
+// GPT-J those of the whole rotated span.
+// Everything the first loads need sits in the first 56 bytes of the kernel arguments, which the
+// hardware preloads into scalar registers at wave launch.
+struct RopeLaunch {
+  const int64_t* positions;
+  void* a;
+  const void* cache;
+  int64_t a_stride_bytes;
+  int64_t delta0;
+  int64_t delta_step;
+  uint32_t geom;
+  uint32_t heads;
+};
+constexpr uint32_t kRopeAIsKey = 0x80000000u;
+
+// One wave: SPW consecutive segments of one token.  FLAT: the launch is one-dimensional with one
+// wave per token (a (1, tokens) grid dispatches measurably slower than a (tokens) grid);
+// otherwise grid = (chunks, tokens) and chunk c is segments [c * SPW, (c + 1) * SPW).
+// The position is a scalar load that the compiler places behind the data loads; moving it, or the
+// cos/sin loads that depend on it, ahead of them measured 5-10 % slower.
+//
+// APPEND: the rotary embedding fused with the paged KV-cache append.  The reference rotates q and
+// k in place (models/llama.py:178) and then copies k and v into the paged cache with flashinfer's
+// append_paged_kv_cache (attention/flashinfer_attention_wrapper.py:262-273).  Fused, the rotated k
+// goes straight from registers to its cache entry (k is read once and, unless the caller asks for
+// the in-place result too, written once), and the v row is copied by the same wave: with
+// rot_dim == head_size, which this path requires, the x and y vectors of a k segment cover its
+// heads completely, so the v vectors at the same two offsets cover the same heads of the v row.
+// The entry address is resolved with scalar loads while the data loads are in flight.
+template <int DT, bool NEOX, int SPW, bool FLAT, bool APPEND>
+SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
+                      const void* __restrict__ cache, int64_t a_stride_bytes, int64_t delta0,
+                      int64_t delta_step, uint32_t geom, uint32_t heads,
+                      const void* __restrict__ value, int64_t v_stride_bytes, uint32_t write_key,
+                      const KvDest* d) {
+  constexpr int SP = SPW == 1 ? kStreamStore : kNtStore;
+  const uint32_t head_bytes = geom & 0xffffu, embed_bytes = geom >> 16;
+  const uint32_t heads_a = heads & 0xfffu, heads_b = (heads >> 12) & 0xfffu;
+  const uint32_t sh = (heads >> 24) & 0x7fu;
+  const bool a_is_key = (heads & kRopeAIsKey) != 0;
+  const int64_t tok = FLAT ? (int64_t)blockIdx.x : (int64_t)blockIdx.z * kMaxGridY + blockIdx.y;
+  const uint32_t chunk = FLAT ? 0u : blockIdx.x;
+  const uint32_t delta = (uint32_t)(delta0 + tok * delta_step);
+  // A's row and, beyond it, B's: per-access validity is decided below (kClipped), the resource
+  // only has to reach past B's row
+  const rsrc_t r = make_rsrc(reinterpret_cast<char*>(a) + tok * a_stride_bytes, 0x7fffffffu);
+  const uint32_t a_pad = (((heads_a << sh) + 63u) >> 6) << (6 - sh);  // A's heads in whole segments
+  const uint32_t slot = threadIdx.x & ((1u << sh) - 1u);
+  const uint32_t h0 = chunk * (uint32_t)(SPW << (6 - sh)) + (threadIdx.x >> sh);
+
+  bool appended = false;
+  if constexpr (APPEND) appended = tok < d->nnz;  // uniform over the wave
+  const uint32_t kv_row_bytes = (a_is_key ? heads_a : heads_b) * head_bytes;
+
+  u32x4 xr[SPW], yr[SPW], vx[SPW], vy[SPW];
+  uint32_t xoff[SPW];   // offset of the lane's x vector from A's row
+  uint32_t koff[SPW];   // APPEND: the same offset inside the k / v row
+#pragma unroll
+  for (int j = 0; j < SPW; ++j) {
+    const uint32_t h = h0 + (uint32_t)(j << (6 - sh));
+    const uint32_t hb = h - a_pad;  // wraps to a huge value while h is inside A's padded span
+    const bool in_a = h < heads_a, in_b = hb < heads_b;
+    const uint32_t row_off = (in_a ? h : hb) * head_bytes + slot * 16u;
+    xoff[j] = (in_a || in_b) ? row_off + (in_a ? 0u : delta) : kClipped;
+    xr[j] = buf_load16<kStreamLoad>(r, xoff[j]);
+    if constexpr (NEOX) yr[j] = buf_load16<kStreamLoad>(r, xoff[j] + embed_bytes);
+    if constexpr (APPEND) {
+      // a segment lies wholly in A's padded span or wholly in B's: uniform
+      const bool seg_in_a = (chunk * SPW + j) < (a_pad >> (6 - sh));
+      const bool is_k = seg_in_a == a_is_key;
+      koff[j] = (in_a || in_b) ? row_off : kClipped;
+      if (is_k && appended) {
+        const rsrc_t rv = make_rsrc(
+            reinterpret_cast<const char*>(value) + tok * v_stride_bytes, kv_row_bytes);
+        vx[j] = buf_load16<kStreamLoad>(rv, koff[j]);
+        if constexpr (NEOX) vy[j] = buf_load16<kStreamLoad>(rv, koff[j] + embed_bytes);
+      }
+    }
+  }
+  // everything above is issued before the first wait (the position's)
   __builtin_amdgcn_sched_barrier(0);
   const rsrc_t rc = make_rsrc(
       reinterpret_cast<const char*>(cache) + positions[tok] * (int64_t)(2 * embed_bytes),
       2 * embed_bytes);
-
   u32x4 cr, sr;
   if constexpr (NEOX) {
     cr = buf_load16<kCached>(rc, slot * 16u);
@@ -91,33 +197,113 @@ __global__ __launch_bounds__(64) void rope_seg_kernel(
     cr = (u32x4){c2.x, c2.y, 0, 0};
     sr = (u32x4){s2.x, s2.y, 0, 0};
   }
-  // all four loads are in flight before the first result is waited for
+  // destination of the k and v rows: resolved while the data loads are in flight
+  int64_t entry = 0;
+  if constexpr (APPEND) {
+    if (appended) entry = kv_entry_offset(*d, tok);
+  }
   __builtin_amdgcn_sched_barrier(0);
 
-  Vec<DT> x, c, s;
-  x.unpack(xr);
+  Vec<DT> c, s;
   c.unpack(cr);
   s.unpack(sr);
-  if constexpr (NEOX) {
-    Vec<DT> y, ox, oy;
-    y.unpack(yr);
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-      ox.f[i] = mul_r<DT>(x.f[i], c.f[i]) - mul_r<DT>(y.f[i], s.f[i]);
-      oy.f[i] = mul_r<DT>(y.f[i], c.f[i]) + mul_r<DT>(x.f[i], s.f[i]);
+  for (int j = 0; j < SPW; ++j) {
+    rotate_slot<DT, NEOX>(xr[j], yr[j], c, s);
+    bool in_place = true;
+    if constexpr (APPEND) {
+      const bool seg_in_a = (chunk * SPW + j) < (a_pad >> (6 - sh));
+      const bool is_k = seg_in_a == a_is_key;
+      in_place = !is_k || write_key != 0 || !appended;
+      if (is_k && appended) {  // uniform
+        const rsrc_t rkc = make_rsrc(reinterpret_cast<char*>(d->k_cache) + entry, kv_row_bytes);
+        const rsrc_t rvc = make_rsrc(reinterpret_cast<char*>(d->v_cache) + entry, kv_row_bytes);
+        buf_store16<kKvStore>(rkc, koff[j], xr[j]);
+        if constexpr (NEOX) buf_store16<kKvStore>(rkc, koff[j] + embed_bytes, yr[j]);
+        buf_store16<kKvStore>(rvc, koff[j], vx[j]);
+        if constexpr (NEOX) buf_store16<kKvStore>(rvc, koff[j] + embed_bytes, vy[j]);
+      }
     }
-    buf_store16<kStreamStore>(rd, xoff, ox.pack());
-    buf_store16<kStreamStore>(rd, xoff + embed_bytes, oy.pack());
-  } else {
-    Vec<DT> o;
-#pragma unroll
-    for (int i = 0; i < N / 2; ++i) {
-      const float xe = x.f[2 * i], ye = x.f[2 * i + 1];
-      o.f[2 * i] = mul_r<DT>(xe, c.f[i]) - mul_r<DT>(ye, s.f[i]);
-      o.f[2 * i + 1] = mul_r<DT>(ye, c.f[i]) + mul_r<DT>(xe, s.f[i]);
+    if (in_place) {
+      buf_store16<SP>(r, xoff[j], xr[j]);
+      if constexpr (NEOX) buf_store16<SP>(r, xoff[j] + embed_bytes, yr[j]);
     }
-    buf_store16<kStreamStore>(rd, xoff, o.pack());
   }
+}
+
+template <int DT, bool NEOX, int SPW, bool FLAT>
+__global__ __launch_bounds__(64) void rope_tok_kernel(
+    const int64_t* __restrict__ positions, void* a, const void* __restrict__ cache,
+    int64_t a_stride_bytes, int64_t delta0, int64_t delta_step, uint32_t geom, uint32_t heads) {
+  rope_wave<DT, NEOX, SPW, FLAT, false>(positions, a, cache, a_stride_bytes, delta0, delta_step,
+                                        geom, heads, nullptr, 0, 0, nullptr);
+}
+
+template <int DT, bool NEOX, int SPW, bool FLAT>
+__global__ __launch_bounds__(64) void rope_append_tok_kernel(
+    const int64_t* __restrict__ positions, void* a, const void* __restrict__ cache,
+    int64_t a_stride_bytes, int64_t delta0, int64_t delta_step, uint32_t geom, uint32_t heads,
+    const void* __restrict__ value, int64_t v_stride_bytes, uint32_t write_key, KvDest d) {
+  rope_wave<DT, NEOX, SPW, FLAT, true>(positions, a, cache, a_stride_bytes, delta0, delta_step,
+                                       geom, heads, value, v_stride_bytes, write_key, &d);
+}
+
+// Segments a wave takes: the whole token when it has at most kMaxSegsPerWave, otherwise the
+// token's list is cut into equal chunks.
+constexpr int kMaxSegsPerWave = 5;
+struct RopeChunks {
+  int chunks, spw;
+};
+static RopeChunks plan_rope_chunks(int64_t segs) {
+  RopeChunks p;
+  p.chunks = (int)((segs + kMaxSegsPerWave - 1) / kMaxSegsPerWave);
+  if (p.chunks < 1) p.chunks = 1;
+  p.spw = (int)((segs + p.chunks - 1) / p.chunks);
+  if (p.spw < 1) p.spw = 1;
+  return p;
+}
+
+// How query and key rows map onto the A / B arrays of a launch.  `pieces` is 1 when B can be
+// reached through A's resource for every token, else 2 (query alone, then key alone).
+struct RopeAnchor {
+  int pieces;
+  RopeLaunch l[2];
+  int64_t segs[2];
+};
+static RopeAnchor plan_rope_anchor(const RopeArgs& a, int eb, int slots, int slot_shift,
+                                   uint32_t geom) {
+  const int64_t qsb = a.q_stride * eb, ksb = a.k_stride * eb;
+  const int64_t q_row = (int64_t)a.num_heads * a.head_size * eb;
+  const int64_t k_row = (int64_t)a.num_kv_heads * a.head_size * eb;
+  char* q = reinterpret_cast<char*>(a.query);
+  char* k = reinterpret_cast<char*>(a.key);
+  const int64_t last = a.num_tokens - 1;
+  const int64_t d_first = k - q, d_last = d_first + last * (ksb - qsb);  // key row - query row
+  const int64_t q_blocks = ((int64_t)a.num_heads * slots + 63) / 64;
+  const int64_t k_blocks = ((int64_t)a.num_kv_heads * slots + 63) / 64;
+  const int64_t reach = (int64_t)kClipped - 64;  // offsets, + embed_bytes, must stay below kClipped
+  const uint32_t sh = (uint32_t)slot_shift << 24;
+  RopeAnchor p;
+  if (a.num_kv_heads == 0 || (d_first >= 0 && d_last >= 0 && d_first + k_row < reach &&
+                              d_last + k_row < reach)) {
+    p.pieces = 1;  // A = query, B = key
+    p.l[0] = {a.positions, q, a.cache, qsb, d_first, ksb - qsb, geom,
+              (uint32_t)a.num_heads | ((uint32_t)a.num_kv_heads << 12) | sh};
+    p.segs[0] = q_blocks + k_blocks;
+  } else if (d_first <= 0 && d_last <= 0 && -d_first + q_row < reach && -d_last + q_row < reach) {
+    p.pieces = 1;  // A = key, B = query
+    p.l[0] = {a.positions, k, a.cache, ksb, -d_first, qsb - ksb, geom,
+              (uint32_t)a.num_kv_heads | ((uint32_t)a.num_heads << 12) | sh | kRopeAIsKey};
+    p.segs[0] = q_blocks + k_blocks;
+  } else {
+    p.pieces = 2;  // too far apart (or crossing): each array on its own
+    p.l[0] = {a.positions, q, a.cache, qsb, 0, 0, geom, (uint32_t)a.num_heads | sh};
+    p.segs[0] = q_blocks;
+    p.l[1] = {a.positions, k, a.cache, ksb, 0, 0, geom,
+              (uint32_t)a.num_kv_heads | sh | kRopeAIsKey};
+    p.segs[1] = k_blocks;
+  }
+  return p;
 }
 
 // Any alignment / rot_dim: one thread per rotated pair, one block per token.
@@ -140,6 +326,70 @@ __global__ __launch_bounds__(256) void rope_generic_kernel(RopeArgs a) {
     store_elem<DT>(arr, xi, mul_r<DT>(x, c) - mul_r<DT>(y, s));
     store_elem<DT>(arr, yi, mul_r<DT>(y, c) + mul_r<DT>(x, s));
   }
+}
+
+// Launches the wave kernels for one piece of an anchor plan.  One wave per token goes out as a
+// one-dimensional grid; chunked tokens as (chunks, tokens), with tokens above 65535 spilling into
+// grid.z and the ragged remainder launched apart.
+template <int DT, bool NEOX, bool APPEND>
+static int launch_rope_piece(const RopeLaunch& l, int64_t segs, int64_t num_tokens,
+                             const void* value, int64_t vsb, int write_key, const KvDest* d,
+                             hipStream_t st) {
+  if (segs <= 0) return SARATHI_OK;
+  const RopeChunks plan = plan_rope_chunks(segs);
+  const bool flat = plan.chunks == 1;
+  const int64_t full_z = flat ? 0 : num_tokens / kMaxGridY;
+  const int64_t rem = flat ? num_tokens : num_tokens % kMaxGridY;
+  const int64_t t0 = full_z * kMaxGridY;
+  // arguments of the remainder launch: everything indexed by token moves on by t0
+  RopeLaunch lr = l;
+  lr.positions += t0;
+  lr.a = reinterpret_cast<char*>(l.a) + t0 * l.a_stride_bytes;
+  lr.delta0 += t0 * l.delta_step;
+  KvDest d0{}, dr{};
+  const void* value_r = value;
+  if constexpr (APPEND) {
+    d0 = *d;
+    dr = *d;
+    if (dr.slot_mapping) {
+      dr.slot_mapping += t0;
+    } else {
+      dr.batch_indices += t0;
+      dr.positions += t0;
+    }
+    dr.nnz = d->nnz > t0 ? d->nnz - t0 : 0;
+    value_r = reinterpret_cast<const char*>(value) + t0 * vsb;
+  }
+  const dim3 block(64);
+  const dim3 grid_full((unsigned)plan.chunks, kMaxGridY, (unsigned)full_z);
+  const dim3 grid_rem = flat ? dim3((unsigned)rem) : dim3((unsigned)plan.chunks, (unsigned)rem, 1);
+#define SK_ROPE_GO(SPW, FLAT, GRID, L, VALUE, DEST)                                              \
+  do {                                                                                           \
+    if constexpr (APPEND)                                                                        \
+      hipLaunchKernelGGL((rope_append_tok_kernel<DT, NEOX, SPW, FLAT>), GRID, block, 0, st,      \
+                         L.positions, L.a, L.cache, L.a_stride_bytes, L.delta0, L.delta_step,    \
+                         L.geom, L.heads, VALUE, vsb, (uint32_t)write_key, DEST);                \
+    else                                                                                         \
+      hipLaunchKernelGGL((rope_tok_kernel<DT, NEOX, SPW, FLAT>), GRID, block, 0, st,             \
+                         L.positions, L.a, L.cache, L.a_stride_bytes, L.delta0, L.delta_step,    \
+                         L.geom, L.heads);                                                       \
+  } while (0)
+#define SK_ROPE_LAUNCH(SPW)                                                \
+  case SPW:                                                                \
+    if (flat) {                                                            \
+      SK_ROPE_GO(SPW, true, grid_rem, lr, value_r, dr);                    \
+    } else {                                                               \
+      if (full_z > 0) SK_ROPE_GO(SPW, false, grid_full, l, value, d0);     \
+      if (rem > 0) SK_ROPE_GO(SPW, false, grid_rem, lr, value_r, dr);      \
+    }                                                                      \
+    break;
+  switch (plan.spw) {
+    SK_ROPE_LAUNCH(1) SK_ROPE_LAUNCH(2) SK_ROPE_LAUNCH(3) SK_ROPE_LAUNCH(4) SK_ROPE_LAUNCH(5)
+    default: return SARATHI_ERR_UNSUPPORTED;
+  }
+#undef SK_ROPE_LAUNCH
+#undef SK_ROPE_GO
+  return launch_status();
 }
 
 template <int DT, bool NEOX>
@@ -167,8 +417,11 @@ static int launch_rope(const RopeArgs& a, hipStream_t st) {
   int slot_shift = 0;
   while ((1 << slot_shift) < slots) ++slot_shift;
   const int64_t head_bytes = (int64_t)a.head_size * EB;
-  // the packed-argument kernel needs power-of-two slots and fields that fit their bit widths
-  const bool packable = (1 << slot_shift) == slots && head_bytes < 65536 && embed * EB < 65536 &&
+  // the packed-argument kernel needs a power-of-two number of slots per head, at most a wave's
+  // worth (so a lane keeps its slot, hence its cos/sin vectors, across segments), and fields that
+  // fit their bit widths
+  const bool packable = (1 << slot_shift) == slots && slots <= 64 && head_bytes < 65536 &&
+                        embed * EB < 65536 &&
                         a.num_heads < 4096 && a.num_kv_heads < 4096;
   if (!packable) {
     hipLaunchKernelGGL((rope_generic_kernel<DT, NEOX>), dim3((unsigned)a.num_tokens), dim3(256),
@@ -176,130 +429,17 @@ static int launch_rope(const RopeArgs& a, hipStream_t st) {
     return launch_status();
   }
   const uint32_t geom = (uint32_t)head_bytes | ((uint32_t)(embed * EB) << 16);
-  const uint32_t heads =
-      (uint32_t)a.num_heads | ((uint32_t)a.num_kv_heads << 12) | ((uint32_t)slot_shift << 24);
-  const int64_t q_blocks = ((int64_t)a.num_heads * slots + 63) / 64;
-  const int64_t k_blocks = ((int64_t)a.num_kv_heads * slots + 63) / 64;
-  const unsigned gx = (unsigned)(q_blocks + k_blocks);
-  const int64_t qsb = a.q_stride * EB, ksb = a.k_stride * EB;
-  // tokens above 65535 spill into grid.z; the ragged remainder is launched apart
-  const int64_t full_z = a.num_tokens / kMaxGridY, rem = a.num_tokens % kMaxGridY;
-  if (full_z > 0)
-    hipLaunchKernelGGL((rope_seg_kernel<DT, NEOX>), dim3(gx, kMaxGridY, (unsigned)full_z), dim3(64),
-                       0, st, a.positions, a.query, a.key, a.cache, qsb, ksb, geom, heads);
-  if (rem > 0) {
-    const int64_t t0 = full_z * kMaxGridY;
-    hipLaunchKernelGGL((rope_seg_kernel<DT, NEOX>), dim3(gx, (unsigned)rem, 1), dim3(64), 0, st,
-                       a.positions + t0, reinterpret_cast<char*>(a.query) + t0 * qsb,
-                       reinterpret_cast<char*>(a.key) + t0 * ksb, a.cache, qsb, ksb, geom, heads);
+  const RopeAnchor plan = plan_rope_anchor(a, EB, slots, slot_shift, geom);
+  for (int i = 0; i < plan.pieces; ++i) {
+    const int rc = launch_rope_piece<DT, NEOX, false>(plan.l[i], plan.segs[i], a.num_tokens,
+                                                      nullptr, 0, 0, nullptr, st);
+    if (rc != SARATHI_OK) return rc;
   }
-  return launch_status();
+  return SARATHI_OK;
 }
 
-// ---- rotary embedding fused with the paged KV-cache append -------------------------------------
+// ---- rotary embedding fused with the paged KV-cache append: element-wise fallback ------------
 //
-// The reference rotates q and k in place (models/llama.py:178) and then copies k and v into the
-// paged cache with flashinfer's append_paged_kv_cache (attention/flashinfer_attention_wrapper.py:
-// 262-273).  Fused, the rotated k goes straight from registers to its cache entry (k is read once
-// and, unless the caller asks for the in-place result too, written once), and v is copied by the
-// same launch.  Workgroup ids run over the q segments, the k segments and then the 16-byte pieces
-// of the v row of one token.  Needs rot_dim == head_size (so the rotated span is the whole head).
-template <int DT, bool NEOX>
-__global__ __launch_bounds__(64) void rope_append_seg_kernel(
-    void* query, void* key, const void* __restrict__ value, uint32_t q_stride_bytes,
-    uint32_t k_stride_bytes, uint32_t v_stride_bytes, uint32_t geom, uint32_t heads,
-    uint32_t write_key, const int64_t* __restrict__ positions, const void* __restrict__ cache,
-    KvDest d) {
-  constexpr int N = VecElems<DT>::value;
-  const uint32_t head_bytes = geom & 0xffffu, embed_bytes = geom >> 16;
-  const int num_heads = heads & 0xfffu, num_kv_heads = (heads >> 12) & 0xfffu;
-  const int slot_shift = heads >> 24;
-  const int q_blocks = ((num_heads << slot_shift) + 63) >> 6;
-  const int k_blocks = ((num_kv_heads << slot_shift) + 63) >> 6;
-  const int64_t tok = (int64_t)blockIdx.z * kMaxGridY + blockIdx.y;
-  const uint32_t kv_row_bytes = (uint32_t)num_kv_heads * head_bytes;
-  const bool appended = tok < d.nnz;  // uniform over the wave
-
-  if ((int)blockIdx.x >= q_blocks + k_blocks) {  // a piece of the v row: plain copy
-    if (!appended) return;
-    const uint32_t off = (((int)blockIdx.x - q_blocks - k_blocks) * 64u + threadIdx.x) * 16u;
-    const char* src = reinterpret_cast<const char*>(value) + tok * (int64_t)v_stride_bytes;
-    const u32x4 v = buf_load16<kStreamLoad>(make_rsrc(src, kv_row_bytes), off);
-    char* dst = reinterpret_cast<char*>(d.v_cache) + kv_entry_offset(d, tok);
-    buf_store16<kKvStore>(make_rsrc(dst, kv_row_bytes), off, v);
-    return;
-  }
-
-  const bool is_q = (int)blockIdx.x < q_blocks;
-  const int item = ((int)blockIdx.x - (is_q ? 0 : q_blocks)) * 64 + (int)threadIdx.x;
-  const int nheads = is_q ? num_heads : num_kv_heads;
-  const int h = item >> slot_shift;
-  const uint32_t slot = item & ((1 << slot_shift) - 1);
-  char* base = reinterpret_cast<char*>(is_q ? query : key) +
-               tok * (int64_t)(is_q ? q_stride_bytes : k_stride_bytes);
-  const rsrc_t rd = make_rsrc(base, (uint32_t)nheads * head_bytes);
-  const uint32_t xoff = h < nheads ? (uint32_t)h * head_bytes + slot * 16u : kClipped;
-
-  u32x4 xr, yr;
-  xr = buf_load16<kStreamLoad>(rd, xoff);
-  if constexpr (NEOX) yr = buf_load16<kStreamLoad>(rd, xoff + embed_bytes);
-  __builtin_amdgcn_sched_barrier(0);
-  const rsrc_t rc = make_rsrc(
-      reinterpret_cast<const char*>(cache) + positions[tok] * (int64_t)(2 * embed_bytes),
-      2 * embed_bytes);
-  u32x4 cr, sr;
-  if constexpr (NEOX) {
-    cr = buf_load16<kCached>(rc, slot * 16u);
-    sr = buf_load16<kCached>(rc, embed_bytes + slot * 16u);
-  } else {
-    const u32x2 c2 = buf_load8<kCached>(rc, slot * 8u);
-    const u32x2 s2 = buf_load8<kCached>(rc, embed_bytes + slot * 8u);
-    cr = (u32x4){c2.x, c2.y, 0, 0};
-    sr = (u32x4){s2.x, s2.y, 0, 0};
-  }
-  // destination of a k segment: resolved while the data loads are in flight
-  const bool to_cache = !is_q && appended;
-  rsrc_t rk = rd;
-  if (to_cache)
-    rk = make_rsrc(reinterpret_cast<char*>(d.k_cache) + kv_entry_offset(d, tok), kv_row_bytes);
-  const bool in_place = is_q || write_key != 0 || !appended;
-  __builtin_amdgcn_sched_barrier(0);
-
-  Vec<DT> x, c, s;
-  x.unpack(xr);
-  c.unpack(cr);
-  s.unpack(sr);
-  if constexpr (NEOX) {
-    Vec<DT> y, ox, oy;
-    y.unpack(yr);
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-      ox.f[i] = mul_r<DT>(x.f[i], c.f[i]) - mul_r<DT>(y.f[i], s.f[i]);
-      oy.f[i] = mul_r<DT>(y.f[i], c.f[i]) + mul_r<DT>(x.f[i], s.f[i]);
-    }
-    const u32x4 px = ox.pack(), py = oy.pack();
-    if (in_place) {
-      buf_store16<kStreamStore>(rd, xoff, px);
-      buf_store16<kStreamStore>(rd, xoff + embed_bytes, py);
-    }
-    if (to_cache) {
-      buf_store16<kKvStore>(rk, xoff, px);
-      buf_store16<kKvStore>(rk, xoff + embed_bytes, py);
-    }
-  } else {
-    Vec<DT> o;
-#pragma unroll
-    for (int i = 0; i < N / 2; ++i) {
-      const float xe = x.f[2 * i], ye = x.f[2 * i + 1];
-      o.f[2 * i] = mul_r<DT>(xe, c.f[i]) - mul_r<DT>(ye, s.f[i]);
-      o.f[2 * i + 1] = mul_r<DT>(ye, c.f[i]) + mul_r<DT>(xe, s.f[i]);
-    }
-    const u32x4 po = o.pack();
-    if (in_place) buf_store16<kStreamStore>(rd, xoff, po);
-    if (to_cache) buf_store16<kKvStore>(rk, xoff, po);
-  }
-}
-
 // Any alignment / rot_dim < head_size: one workgroup per token.
 template <int DT, bool NEOX>
 __global__ __launch_bounds__(256) void rope_append_generic_kernel(RopeArgs a, const void* value,
@@ -369,8 +509,8 @@ static int launch_rope_append(const RopeArgs& a, const void* value, int64_t v_st
       aligned16(a.query) && aligned16(a.key) && aligned16(value) && aligned16(a.cache) &&
       aligned16(d.k_cache) && aligned16(d.v_cache) && d.page_stride_bytes % 16 == 0 &&
       d.entry_stride_bytes % 16 == 0 && q_row_bytes < (int64_t)kClipped &&
-      k_row_bytes < (int64_t)kClipped && qsb < (1LL << 32) && ksb < (1LL << 32) &&
-      vsb < (1LL << 32) && (1 << slot_shift) == slots && head_bytes < 65536 &&
+      k_row_bytes < (int64_t)kClipped && (1 << slot_shift) == slots && slots <= 64 &&
+      head_bytes < 65536 &&
       embed * EB < 65536 && a.num_heads < 4096 && a.num_kv_heads < 4096;
   if (!vec_ok) {
     hipLaunchKernelGGL((rope_append_generic_kernel<DT, NEOX>), dim3((unsigned)a.num_tokens),
@@ -378,35 +518,13 @@ static int launch_rope_append(const RopeArgs& a, const void* value, int64_t v_st
     return launch_status();
   }
   const uint32_t geom = (uint32_t)head_bytes | ((uint32_t)(embed * EB) << 16);
-  const uint32_t heads =
-      (uint32_t)a.num_heads | ((uint32_t)a.num_kv_heads << 12) | ((uint32_t)slot_shift << 24);
-  const int64_t q_blocks = ((int64_t)a.num_heads * slots + 63) / 64;
-  const int64_t k_blocks = ((int64_t)a.num_kv_heads * slots + 63) / 64;
-  const int64_t v_blocks = (k_row_bytes / 16 + 63) / 64;
-  const unsigned gx = (unsigned)(q_blocks + k_blocks + v_blocks);
-  const int64_t full_z = a.num_tokens / kMaxGridY, rem = a.num_tokens % kMaxGridY;
-  if (full_z > 0)
-    hipLaunchKernelGGL((rope_append_seg_kernel<DT, NEOX>), dim3(gx, kMaxGridY, (unsigned)full_z),
-                       dim3(64), 0, st, a.query, a.key, value, (uint32_t)qsb, (uint32_t)ksb,
-                       (uint32_t)vsb, geom, heads, (uint32_t)write_key, a.positions, a.cache, d);
-  if (rem > 0) {
-    const int64_t t0 = full_z * kMaxGridY;
-    KvDest dr = d;
-    if (dr.slot_mapping) {
-      dr.slot_mapping += t0;
-    } else {
-      dr.batch_indices += t0;
-      dr.positions += t0;
-    }
-    dr.nnz = d.nnz > t0 ? d.nnz - t0 : 0;
-    hipLaunchKernelGGL((rope_append_seg_kernel<DT, NEOX>), dim3(gx, (unsigned)rem, 1), dim3(64), 0,
-                       st, reinterpret_cast<char*>(a.query) + t0 * qsb,
-                       reinterpret_cast<char*>(a.key) + t0 * ksb,
-                       reinterpret_cast<const char*>(value) + t0 * vsb, (uint32_t)qsb,
-                       (uint32_t)ksb, (uint32_t)vsb, geom, heads, (uint32_t)write_key,
-                       a.positions + t0, a.cache, dr);
+  const RopeAnchor plan = plan_rope_anchor(a, EB, slots, slot_shift, geom);
+  for (int i = 0; i < plan.pieces; ++i) {
+    const int rc = launch_rope_piece<DT, NEOX, true>(plan.l[i], plan.segs[i], a.num_tokens, value,
+                                                     vsb, write_key, &d, st);
+    if (rc != SARATHI_OK) return rc;
   }
-  return launch_status();
+  return SARATHI_OK;
 }
 
 }  // namespace sarathi_hip
