@@ -91,6 +91,121 @@ __global__ __launch_bounds__(64 * WAVES) void rms_norm_row_kernel(
   }
 }
 
+// fused_add_rms_norm with R consecutive rows per workgroup: the loads of all R rows are issued
+// up front, the weight vectors are fetched and unpacked once for the R rows, and the launch has
+// R times fewer workgroups.  At mid-sized batches that is worth 6 % (2304 rows of 4096 bf16 on
+// MI355X: 13.8 us with one row per workgroup, 12.9 us with three) provided the workgroups divide
+// evenly over the compute units; pick_rows_per_workgroup() decides.  Rows at or beyond num_rows
+// get an empty buffer resource: their loads return zeros and their stores are dropped.
+template <int DT, int WAVES, int VPL, int R>
+__global__ __launch_bounds__(64 * WAVES) void fused_add_rms_norm_rows_kernel(
+    void* out, void* residual, const void* __restrict__ weight, float eps, uint32_t row_bytes,
+    float hidden_f, int64_t out_stride_bytes, int64_t res_stride_bytes, int64_t num_rows) {
+  constexpr int N = VecElems<DT>::value;
+  constexpr int TPR = 64 * WAVES;
+  __shared__ float partial[R][WAVES];
+  const int64_t row0 = (int64_t)blockIdx.x * R;
+  const rsrc_t rw = make_rsrc(weight, row_bytes);
+  const uint32_t off0 = threadIdx.x * 16u;
+  rsrc_t rres[R], rout[R];
+  u32x4 raw[R][VPL], hid[R][VPL];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const uint32_t live = row0 + r < num_rows ? row_bytes : 0u;
+    rres[r] = make_rsrc(reinterpret_cast<char*>(residual) + (row0 + r) * res_stride_bytes, live);
+    rout[r] = make_rsrc(reinterpret_cast<char*>(out) + (row0 + r) * out_stride_bytes, live);
+#pragma unroll
+    for (int j = 0; j < VPL; ++j)
+      raw[r][j] = buf_load16<kStreamLoad>(rres[r], off0 + j * (TPR * 16u));
+#pragma unroll
+    for (int j = 0; j < VPL; ++j)
+      hid[r][j] = buf_load16<kStreamLoad>(rout[r], off0 + j * (TPR * 16u));
+  }
+  u32x4 wraw[VPL];
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) wraw[j] = buf_load16<kCached>(rw, off0 + j * (TPR * 16u));
+  __builtin_amdgcn_sched_barrier(0);  // every load is issued before the first wait
+
+  float ss[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    ss[r] = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      Vec<DT> a, b;
+      a.unpack(raw[r][j]);
+      b.unpack(hid[r][j]);
+#pragma unroll
+      for (int i = 0; i < N; ++i) a.f[i] = b.f[i] + a.f[i];
+      raw[r][j] = a.pack();  // z, rounded to the dtype
+      buf_store16<kStreamStore>(rres[r], off0 + j * (TPR * 16u), raw[r][j]);
+      a.unpack(raw[r][j]);
+#pragma unroll
+      for (int i = 0; i < N; ++i) ss[r] = __builtin_fmaf(a.f[i], a.f[i], ss[r]);
+    }
+    ss[r] = wave64_sum(ss[r]);
+    if constexpr (WAVES > 1) {
+      if ((threadIdx.x & 63) == 0) partial[r][threadIdx.x >> 6] = ss[r];
+    }
+  }
+  if constexpr (WAVES > 1) lds_barrier();  // the residual stores above stay in flight
+  Vec<DT> w[VPL];
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) w[j].unpack(wraw[j]);
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if constexpr (WAVES > 1) {
+      float t = partial[r][0];
+#pragma unroll
+      for (int k = 1; k < WAVES; ++k) t += partial[r][k];
+      ss[r] = t;
+    }
+    const float s = __builtin_amdgcn_rsqf(ss[r] / hidden_f + eps);
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      Vec<DT> a;
+      a.unpack(raw[r][j]);
+#pragma unroll
+      for (int i = 0; i < N; i += 2) {
+        const f32x2 t = rnd2<DT>(a.f[i] * s, a.f[i + 1] * s);
+        a.f[i] = t.x * w[j].f[i];
+        a.f[i + 1] = t.y * w[j].f[i + 1];
+      }
+      buf_store16<kStreamStore>(rout[r], off0 + j * (TPR * 16u), a.pack());
+    }
+  }
+}
+
+// Rows per workgroup for the kernel above.  Workgroups are dealt to the compute units in turn, so
+// the launch lasts as long as the busiest unit: ceil(workgroups / units) * R rows.  Take the
+// largest R (fewest weight fetches, fewest workgroups) among those with the shortest busiest
+// unit, but keep one row per workgroup while that leaves fewer than two workgroups per unit
+// (small batches need the parallelism more).
+static int pick_rows_per_workgroup(int64_t rows, int max_rows_per_wg) {
+  static const int units = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        n <= 0) {
+      (void)hipGetLastError();
+      n = 256;
+    }
+    return n;
+  }();
+  int best = 1;
+  int64_t best_cost = (rows + units - 1) / units;
+  for (int r = 2; r <= max_rows_per_wg; ++r) {
+    const int64_t wgs = (rows + r - 1) / r;
+    if (wgs < 2 * (int64_t)units) break;
+    const int64_t cost = (wgs + units - 1) / units * r;
+    if (cost <= best_cost) {
+      best = r;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+
 // Any shape / alignment: one 256-thread block per row, element-wise accesses,
 // the row re-read from cache for the second pass.
 template <int DT, bool FUSED>
@@ -148,7 +263,19 @@ static int launch_rms(void* out, void* in, const void* w, float eps, int64_t T, 
   else if (nvec <= 128) SK_RMS_CASE(1, 2);
   else if (FUSED) {
     if (nvec <= 256) SK_RMS_CASE(2, 2);
-    else if (nvec <= 512) SK_RMS_CASE(4, 2);
+    else if (nvec <= 512) {
+      // 2 waves x 4 vectors with up to three rows per workgroup where the row count makes that
+      // come out even over the compute units; otherwise 4 waves x 2 vectors, one row
+      const int rows_per_wg = pick_rows_per_workgroup(T, 3);
+      const dim3 rgrid((unsigned)((T + rows_per_wg - 1) / rows_per_wg));
+#define SK_RMS_ROWS(R)                                                                         \
+  hipLaunchKernelGGL((fused_add_rms_norm_rows_kernel<DT, 2, 4, R>), rgrid, dim3(128), 0, st,   \
+                     out, in, w, eps, row_bytes, hidden_f, out_stride * EB, in_stride * EB, T)
+      if (rows_per_wg == 3) SK_RMS_ROWS(3);
+      else if (rows_per_wg == 2) SK_RMS_ROWS(2);
+      else SK_RMS_CASE(4, 2);
+#undef SK_RMS_ROWS
+    }
     else if (nvec <= 1024) SK_RMS_CASE(8, 2);
     else if (nvec <= 2048) SK_RMS_CASE(16, 2);
     else SK_RMS_CASE(16, 4);

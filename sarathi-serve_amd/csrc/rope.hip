@@ -56,15 +56,10 @@ template <int DT> SK_DEV float mul_r(float a, float b) { return rnd<DT>(a * b); 
 // One rotation with the reference's rounding points.  For 16-bit dtypes the two products of each
 // sum go through ONE packed conversion (v_cvt_pk_*) and come back as floats.
 template <int DT> SK_DEV void rotate(float x, float y, float c, float s, float& ox, float& oy) {
-  if constexpr (DT == kF32) {
-    ox = x * c - y * s;
-    oy = y * c + x * s;
-  } else {
-    const f32x2 a = unpack2<DT>(pack2<DT>(x * c, y * s));
-    const f32x2 b = unpack2<DT>(pack2<DT>(y * c, x * s));
-    ox = a.x - a.y;
-    oy = b.x + b.y;
-  }
+  const f32x2 a = rnd2<DT>(x * c, y * s);
+  const f32x2 b = rnd2<DT>(y * c, x * s);
+  ox = a.x - a.y;
+  oy = b.x + b.y;
 }
 
 // Rotates the 16-byte slot(s) of one lane: NeoX x vector `xr` and y vector `yr`; GPT-J only `xr`

@@ -64,6 +64,17 @@ template <> SK_DEV float rnd<kF32>(float f) { return f; }
 template <> SK_DEV float rnd<kBF16>(float f) { return (float)(__bf16)f; }
 template <> SK_DEV float rnd<kF16>(float f) { return (float)(_Float16)f; }
 
+// Round two floats to the tensor dtype and widen again with ONE packed conversion (half the
+// conversions of two rnd<DT>() calls; same results).
+template <int DT> SK_DEV f32x2 rnd2(float a, float b) {
+  if constexpr (DT == kF32) {
+    f32x2 r = {a, b};
+    return r;
+  } else {
+    return unpack2<DT>(pack2<DT>(a, b));
+  }
+}
+
 // ---- a 16-byte vector as an array of floats --------------------------------
 
 template <int DT> struct Vec {

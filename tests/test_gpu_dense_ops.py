@@ -57,6 +57,29 @@ def test_fused_add_rms_norm_matches_oracle(ops, dev, dtype, T, H):
     assert_close_dtype(gx, wx, **_tol(dtype))
 
 
+@pytest.mark.parametrize("T,H", [(2304, 4096), (2305, 4096), (1030, 4096), (2304, 3072),
+                                 (1537, 2560)])
+def test_fused_add_rms_norm_rows_per_workgroup(ops, dev, T, H):
+    """Row counts at which the launch puts two or three rows into one workgroup (2304 -> 3,
+    2305 and 1030 -> 2 with a ragged last workgroup), and widths short of the workgroup's 512
+    vectors: same results as the oracle over every row."""
+    g = gen(T + H)
+    x, r = randn((T, H), g), randn((T, H), g)
+    w = randn((H,), g, mean=1.0, std=0.1)
+    wx, wr = x.clone(), r.clone()
+    c_oracle.fused_add_rms_norm(wx, wr, w, 1e-5)
+    # views into wider buffers: the row stride differs from the width
+    gx_buf = torch.zeros((T, H + 64), dtype=x.dtype, device=dev)
+    gr_buf = torch.zeros((T, H + 8), dtype=x.dtype, device=dev)
+    gx, gr = gx_buf[:, :H], gr_buf[:, :H]
+    gx.copy_(x)
+    gr.copy_(r)
+    ops.layernorm_ops.fused_add_rms_norm(gx, gr, w.to(dev), 1e-5)
+    assert torch.equal(gr.cpu(), wr), "residual = T(x + r) must be bit-exact"
+    assert_close_dtype(gx, wx)
+    assert bool((gx_buf[:, H:] == 0).all()) and bool((gr_buf[:, H:] == 0).all())
+
+
 def test_fused_add_equals_add_then_norm(ops, dev):
     """fused(x, r) == (r' = x + r in bf16; rms_norm(r')) using the library's own rms_norm: the
     fusion changes traffic, not arithmetic.  The residual is bit-exact; the normed output may
