@@ -91,87 +91,76 @@ __global__ __launch_bounds__(64 * WAVES) void rms_norm_row_kernel(
   }
 }
 
-// fused_add_rms_norm with R consecutive rows per workgroup: the loads of all R rows are issued
-// up front, the weight vectors are fetched and unpacked once for the R rows, and the launch has
-// R times fewer workgroups.  At mid-sized batches that is worth 6 % (2304 rows of 4096 bf16 on
-// MI355X: 13.8 us with one row per workgroup, 12.9 us with three) provided the workgroups divide
-// evenly over the compute units; pick_rows_per_workgroup() decides.  Rows at or beyond num_rows
-// get an empty buffer resource: their loads return zeros and their stores are dropped.
-template <int DT, int WAVES, int VPL, int R>
-__global__ __launch_bounds__(64 * WAVES) void fused_add_rms_norm_rows_kernel(
-    void* out, void* residual, const void* __restrict__ weight, float eps, uint32_t row_bytes,
-    float hidden_f, int64_t out_stride_bytes, int64_t res_stride_bytes, int64_t num_rows) {
+// R consecutive rows per one-wave workgroup, for rows of up to 64 * VPL vectors.  The weight
+// vectors are fetched once for the R rows, the loads of all R rows are issued before the first
+// wait, and the rows are then finished one after the other, so row 0 is on its way out while row
+// 2 is still arriving.  The launch has R times fewer workgroups, each with R times the bytes in
+// flight.  On MI355X at 2304 rows of 4096 bf16 (three rows per workgroup = three workgroups per
+// compute unit): fused op 13.8 -> 12.4 us; a plain copy kernel shows the same pattern (2304 waves
+// of 8 KiB each 7.1 us, 768 waves of 24 KiB each 6.4 us).  It only pays
+// when the workgroups divide evenly over the compute units; pick_rows_per_workgroup() decides.
+// Rows at or beyond num_rows get an empty buffer resource: their loads return zeros and their
+// stores are dropped.
+template <int DT, int VPL, int R, bool FUSED>
+__global__ __launch_bounds__(64) void rms_norm_wave_rows_kernel(
+    void* out, void* in_or_res, const void* __restrict__ weight, float eps, uint32_t row_bytes,
+    float hidden_f, int64_t out_stride_bytes, int64_t in_stride_bytes, int64_t num_rows) {
   constexpr int N = VecElems<DT>::value;
-  constexpr int TPR = 64 * WAVES;
-  __shared__ float partial[R][WAVES];
   const int64_t row0 = (int64_t)blockIdx.x * R;
   const rsrc_t rw = make_rsrc(weight, row_bytes);
   const uint32_t off0 = threadIdx.x * 16u;
-  rsrc_t rres[R], rout[R];
+  u32x4 wraw[VPL];
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) wraw[j] = buf_load16<kCached>(rw, off0 + j * 1024u);
+  rsrc_t rin[R], rout[R];
   u32x4 raw[R][VPL], hid[R][VPL];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const uint32_t live = row0 + r < num_rows ? row_bytes : 0u;
-    rres[r] = make_rsrc(reinterpret_cast<char*>(residual) + (row0 + r) * res_stride_bytes, live);
+    rin[r] = make_rsrc(reinterpret_cast<char*>(in_or_res) + (row0 + r) * in_stride_bytes, live);
     rout[r] = make_rsrc(reinterpret_cast<char*>(out) + (row0 + r) * out_stride_bytes, live);
 #pragma unroll
-    for (int j = 0; j < VPL; ++j)
-      raw[r][j] = buf_load16<kStreamLoad>(rres[r], off0 + j * (TPR * 16u));
+    for (int j = 0; j < VPL; ++j) raw[r][j] = buf_load16<kStreamLoad>(rin[r], off0 + j * 1024u);
+    if constexpr (FUSED) {
 #pragma unroll
-    for (int j = 0; j < VPL; ++j)
-      hid[r][j] = buf_load16<kStreamLoad>(rout[r], off0 + j * (TPR * 16u));
+      for (int j = 0; j < VPL; ++j) hid[r][j] = buf_load16<kStreamLoad>(rout[r], off0 + j * 1024u);
+    }
   }
-  u32x4 wraw[VPL];
-#pragma unroll
-  for (int j = 0; j < VPL; ++j) wraw[j] = buf_load16<kCached>(rw, off0 + j * (TPR * 16u));
   __builtin_amdgcn_sched_barrier(0);  // every load is issued before the first wait
 
-  float ss[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    ss[r] = 0.f;
-#pragma unroll
-    for (int j = 0; j < VPL; ++j) {
-      Vec<DT> a, b;
-      a.unpack(raw[r][j]);
-      b.unpack(hid[r][j]);
-#pragma unroll
-      for (int i = 0; i < N; ++i) a.f[i] = b.f[i] + a.f[i];
-      raw[r][j] = a.pack();  // z, rounded to the dtype
-      buf_store16<kStreamStore>(rres[r], off0 + j * (TPR * 16u), raw[r][j]);
-      a.unpack(raw[r][j]);
-#pragma unroll
-      for (int i = 0; i < N; ++i) ss[r] = __builtin_fmaf(a.f[i], a.f[i], ss[r]);
-    }
-    ss[r] = wave64_sum(ss[r]);
-    if constexpr (WAVES > 1) {
-      if ((threadIdx.x & 63) == 0) partial[r][threadIdx.x >> 6] = ss[r];
-    }
-  }
-  if constexpr (WAVES > 1) lds_barrier();  // the residual stores above stay in flight
-  Vec<DT> w[VPL];
-#pragma unroll
-  for (int j = 0; j < VPL; ++j) w[j].unpack(wraw[j]);
-#pragma unroll
-  for (int r = 0; r < R; ++r) {
-    if constexpr (WAVES > 1) {
-      float t = partial[r][0];
-#pragma unroll
-      for (int k = 1; k < WAVES; ++k) t += partial[r][k];
-      ss[r] = t;
-    }
-    const float s = __builtin_amdgcn_rsqf(ss[r] / hidden_f + eps);
+    float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
       Vec<DT> a;
       a.unpack(raw[r][j]);
+      if constexpr (FUSED) {
+        Vec<DT> b;
+        b.unpack(hid[r][j]);
+#pragma unroll
+        for (int i = 0; i < N; ++i) a.f[i] = b.f[i] + a.f[i];
+        raw[r][j] = a.pack();  // z, rounded to the dtype
+        buf_store16<kStreamStore>(rin[r], off0 + j * 1024u, raw[r][j]);
+        a.unpack(raw[r][j]);
+      }
+#pragma unroll
+      for (int i = 0; i < N; ++i) ss = __builtin_fmaf(a.f[i], a.f[i], ss);
+    }
+    ss = wave64_sum(ss);
+    const float s = __builtin_amdgcn_rsqf(ss / hidden_f + eps);
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      Vec<DT> a, w;
+      a.unpack(raw[r][j]);
+      w.unpack(wraw[j]);
 #pragma unroll
       for (int i = 0; i < N; i += 2) {
         const f32x2 t = rnd2<DT>(a.f[i] * s, a.f[i + 1] * s);
-        a.f[i] = t.x * w[j].f[i];
-        a.f[i + 1] = t.y * w[j].f[i + 1];
+        a.f[i] = t.x * w.f[i];
+        a.f[i + 1] = t.y * w.f[i + 1];
       }
-      buf_store16<kStreamStore>(rout[r], off0 + j * (TPR * 16u), a.pack());
+      buf_store16<kStreamStore>(rout[r], off0 + j * 1024u, a.pack());
     }
   }
 }
@@ -180,7 +169,8 @@ __global__ __launch_bounds__(64 * WAVES) void fused_add_rms_norm_rows_kernel(
 // the launch lasts as long as the busiest unit: ceil(workgroups / units) * R rows.  Take the
 // largest R (fewest weight fetches, fewest workgroups) among those with the shortest busiest
 // unit, but keep one row per workgroup while that leaves fewer than two workgroups per unit
-// (small batches need the parallelism more).
+// (small batches need the parallelism more).  Measured at 2304 rows of 4096 bf16: R = 3 (768
+// workgroups, 3 per unit) 12.4 us, R = 2 (1152, i.e. 4.5 per unit) 15.6 us, R = 1 13.8 us.
 static int pick_rows_per_workgroup(int64_t rows, int max_rows_per_wg) {
   static const int units = [] {
     int dev = 0, n = 0;
@@ -255,27 +245,36 @@ static int launch_rms(void* out, void* in, const void* w, float eps, int64_t T, 
 #define SK_RMS_CASE(WAVES, VPL)                                                               \
   hipLaunchKernelGGL((rms_norm_row_kernel<DT, WAVES, VPL, FUSED>), grid, dim3(64 * WAVES), 0, \
                      st, out, in, w, eps, row_bytes, hidden_f, out_stride * EB, in_stride * EB)
-  // Shapes measured on MI355X at H = 4096 and H = 8192 (bf16).  The plain norm is fastest
-  // with a whole row of up to 512 vectors in ONE wave (no LDS, no barrier) and four vectors
-  // per lane beyond that; the fused op, which holds two rows' worth of loads, is fastest with
-  // two vectors per lane and proportionally more waves.
+  // Fused op on rows of 257..512 vectors (H = 4096 at 16 bits): two or three rows per one-wave
+  // workgroup where the row count makes that come out even over the compute units.  (The plain
+  // norm gains nothing from it with write-through stores, 7.1 us either way at 2304 x 4096; with
+  // write-back non-temporal stores it gains 4 % on cold inputs and loses 35 % on inputs that are
+  // still in the memory-side cache, which is how the reference's callers present them.)
+  if (FUSED && nvec > 256 && nvec <= 512) {
+    const int rows_per_wg = pick_rows_per_workgroup(T, 3);
+    const dim3 rgrid((unsigned)((T + rows_per_wg - 1) / rows_per_wg));
+#define SK_RMS_ROWS(R)                                                                           \
+  hipLaunchKernelGGL((rms_norm_wave_rows_kernel<DT, 8, R, FUSED>), rgrid, dim3(64), 0, st, out,  \
+                     in, w, eps, row_bytes, hidden_f, out_stride * EB, in_stride * EB, T)
+    if (rows_per_wg == 3) {
+      SK_RMS_ROWS(3);
+      return launch_status();
+    }
+    if (rows_per_wg == 2) {
+      SK_RMS_ROWS(2);
+      return launch_status();
+    }
+#undef SK_RMS_ROWS
+  }
+  // One row per workgroup.  Shapes measured on MI355X at H = 4096 and H = 8192 (bf16).  The plain
+  // norm is fastest with a whole row of up to 512 vectors in ONE wave (no LDS, no barrier) and
+  // four vectors per lane beyond that; the fused op, which holds two rows' worth of loads, is
+  // fastest with two vectors per lane and proportionally more waves.
   if (nvec <= 64) SK_RMS_CASE(1, 1);
   else if (nvec <= 128) SK_RMS_CASE(1, 2);
   else if (FUSED) {
     if (nvec <= 256) SK_RMS_CASE(2, 2);
-    else if (nvec <= 512) {
-      // 2 waves x 4 vectors with up to three rows per workgroup where the row count makes that
-      // come out even over the compute units; otherwise 4 waves x 2 vectors, one row
-      const int rows_per_wg = pick_rows_per_workgroup(T, 3);
-      const dim3 rgrid((unsigned)((T + rows_per_wg - 1) / rows_per_wg));
-#define SK_RMS_ROWS(R)                                                                         \
-  hipLaunchKernelGGL((fused_add_rms_norm_rows_kernel<DT, 2, 4, R>), rgrid, dim3(128), 0, st,   \
-                     out, in, w, eps, row_bytes, hidden_f, out_stride * EB, in_stride * EB, T)
-      if (rows_per_wg == 3) SK_RMS_ROWS(3);
-      else if (rows_per_wg == 2) SK_RMS_ROWS(2);
-      else SK_RMS_CASE(4, 2);
-#undef SK_RMS_ROWS
-    }
+    else if (nvec <= 512) SK_RMS_CASE(4, 2);
     else if (nvec <= 1024) SK_RMS_CASE(8, 2);
     else if (nvec <= 2048) SK_RMS_CASE(16, 2);
     else SK_RMS_CASE(16, 4);
