@@ -4,8 +4,14 @@
 // (sarathi/model_executor/layers/fused_moe/fused_moe.py:539-543: torch.sum over dim 1 of the
 // [tokens, top_k, hidden] output of the down projection, into the result tensor): fp32
 // accumulation over j in ascending order, one rounding to the tensor dtype.  A streaming op like
-// silu_and_mul and built the same way: one 64-lane workgroup per 1 KiB segment of an output row,
-// top_k 16-byte loads and one 16-byte store per lane, rows as buffer resources.
+// silu_and_mul.  Rows of up to 8 KiB with top_k 1 or 2 (Mixtral) take moe_sum_rows_kernel: ONE wave
+// per R consecutive tokens, all top_k * 8 * R loads issued before the first add, rows as buffer
+// resources, a one-dimensional grid.  Fewer, fatter one-wave workgroups are what the memory
+// system rewards at these sizes (a launch of N one-wave workgroups costs the dispatcher 0.2 ns
+// each, and more bytes in flight per wave hide more of the ramp): the [2304, 1, 4096] case, a
+// plain copy, takes 9.5 us as 18432 one-segment workgroups and 6.4-7.1 us as 768-2304 row waves.
+// Everything else takes the general kernel: one 64-lane workgroup per 1 KiB segment of an output
+// row, top_k 16-byte loads and one 16-byte store per lane.
 #include "vec16.h"
 #include "launch.h"
 
@@ -31,6 +37,50 @@ __global__ __launch_bounds__(kSumSeg) void moe_sum_kernel(
   }
   const rsrc_t ro = make_rsrc(reinterpret_cast<char*>(out) + row * out_stride_bytes, row_bytes);
   buf_store16<kStreamStore>(ro, off, acc.pack());
+}
+
+// One wave per R consecutive tokens; a row has at most 64 * VPL vectors; TOPK is 1 or 2.
+template <int DT, int TOPK, int VPL, int R>
+__global__ __launch_bounds__(kSumSeg) void moe_sum_rows_kernel(
+    void* __restrict__ out, const void* __restrict__ in, uint32_t row_bytes,
+    int64_t in_token_stride_bytes, int64_t in_k_stride_bytes, int64_t out_stride_bytes,
+    int64_t num_rows) {
+  constexpr int N = VecElems<DT>::value;
+  const int64_t row0 = (int64_t)blockIdx.x * R;
+  const uint32_t off0 = threadIdx.x * 16u;
+  u32x4 v[R][TOPK][VPL];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const uint32_t live = row0 + r < num_rows ? row_bytes : 0u;  // rows past the end: no traffic
+    const char* tok = reinterpret_cast<const char*>(in) + (row0 + r) * in_token_stride_bytes;
+#pragma unroll
+    for (int j = 0; j < TOPK; ++j) {
+      const rsrc_t ri = make_rsrc(tok + j * in_k_stride_bytes, live);
+#pragma unroll
+      for (int u = 0; u < VPL; ++u) v[r][j][u] = buf_load16<kStreamLoad>(ri, off0 + u * 1024u);
+    }
+  }
+  // every load is issued before the first wait (left alone, the scheduler starts storing after
+  // ten loads and issues the rest one by one)
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const uint32_t live = row0 + r < num_rows ? row_bytes : 0u;
+    const rsrc_t ro =
+        make_rsrc(reinterpret_cast<char*>(out) + (row0 + r) * out_stride_bytes, live);
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      Vec<DT> acc;
+      acc.unpack(v[r][0][u]);
+      if constexpr (TOPK == 2) {
+        Vec<DT> x;
+        x.unpack(v[r][1][u]);
+#pragma unroll
+        for (int i = 0; i < N; ++i) acc.f[i] += x.f[i];
+      }
+      buf_store16<kStreamStore>(ro, off0 + u * 1024u, acc.pack());
+    }
+  }
 }
 
 template <int DT>
@@ -61,6 +111,33 @@ static int launch_moe_sum(void* out, const void* in, int64_t T, int top_k, int64
     return launch_status();
   }
   const int64_t segs = (hidden / N + kSumSeg - 1) / kSumSeg;
+  if (segs <= 8 && top_k <= 2) {
+    // whole rows per wave; two or three tokens per wave where that divides evenly over the
+    // compute units (top-2: at most two, to stay inside the register file)
+    const int rows = pick_rows_per_workgroup(T, top_k == 1 ? 3 : 2);
+    const dim3 grid((unsigned)((T + rows - 1) / rows));
+    const uint32_t row_bytes = (uint32_t)(hidden * EB);
+#define SK_SUM_ROWS(TOPK, VPL, R)                                                              \
+  hipLaunchKernelGGL((moe_sum_rows_kernel<DT, TOPK, VPL, R>), grid, dim3(kSumSeg), 0, st, out, \
+                     in, row_bytes, in_token_stride * EB, in_k_stride * EB, out_stride * EB, T)
+#define SK_SUM_VPL(TOPK, R)                     \
+  do {                                          \
+    if (segs <= 2) SK_SUM_ROWS(TOPK, 2, R);     \
+    else if (segs <= 4) SK_SUM_ROWS(TOPK, 4, R); \
+    else SK_SUM_ROWS(TOPK, 8, R);               \
+  } while (0)
+    if (top_k == 1) {
+      if (rows == 3) SK_SUM_VPL(1, 3);
+      else if (rows == 2) SK_SUM_VPL(1, 2);
+      else SK_SUM_VPL(1, 1);
+    } else {
+      if (rows == 2) SK_SUM_VPL(2, 2);
+      else SK_SUM_VPL(2, 1);
+    }
+#undef SK_SUM_VPL
+#undef SK_SUM_ROWS
+    return launch_status();
+  }
   // rows above 65535 spill into grid.z; the last z-slice may run past T, so launch it apart
   const int64_t full_z = T / kMaxGridY, rem = T % kMaxGridY;
   const char* inb = reinterpret_cast<const char*>(in);

@@ -165,37 +165,6 @@ __global__ __launch_bounds__(64) void rms_norm_wave_rows_kernel(
   }
 }
 
-// Rows per workgroup for the kernel above.  Workgroups are dealt to the compute units in turn, so
-// the launch lasts as long as the busiest unit: ceil(workgroups / units) * R rows.  Take the
-// largest R (fewest weight fetches, fewest workgroups) among those with the shortest busiest
-// unit, but keep one row per workgroup while that leaves fewer than two workgroups per unit
-// (small batches need the parallelism more).  Measured at 2304 rows of 4096 bf16: R = 3 (768
-// workgroups, 3 per unit) 12.4 us, R = 2 (1152, i.e. 4.5 per unit) 15.6 us, R = 1 13.8 us.
-static int pick_rows_per_workgroup(int64_t rows, int max_rows_per_wg) {
-  static const int units = [] {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-        n <= 0) {
-      (void)hipGetLastError();
-      n = 256;
-    }
-    return n;
-  }();
-  int best = 1;
-  int64_t best_cost = (rows + units - 1) / units;
-  for (int r = 2; r <= max_rows_per_wg; ++r) {
-    const int64_t wgs = (rows + r - 1) / r;
-    if (wgs < 2 * (int64_t)units) break;
-    const int64_t cost = (wgs + units - 1) / units * r;
-    if (cost <= best_cost) {
-      best = r;
-      best_cost = cost;
-    }
-  }
-  return best;
-}
-
 // Any shape / alignment: one 256-thread block per row, element-wise accesses,
 // the row re-read from cache for the second pass.
 template <int DT, bool FUSED>

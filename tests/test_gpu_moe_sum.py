@@ -28,6 +28,19 @@ def test_moe_sum_matches_library_sum(ops, dev, dtype, T, k, H):
         assert_close_dtype(out, want, max_ulps=1)
 
 
+@pytest.mark.parametrize("T,k,H", [(4096, 2, 4096), (4097, 2, 4096), (2304, 1, 4096), (2305, 1, 4096),
+                                   (1030, 1, 1000), (3000, 2, 1536), (2304, 2, 8192)])
+def test_moe_sum_several_tokens_per_wave(ops, dev, T, k, H):
+    """Token counts at which a wave takes two or three tokens (with a ragged last wave), widths
+    short of the wave's span, and a width above it (general kernel): exact for one or two addends."""
+    g = gen(T + k + H)
+    x = randn((T, k, H), g, std=1.5)
+    out_big = torch.full((T + 2, H), 9.0, dtype=x.dtype, device=dev)
+    ops.moe_ops.moe_sum(x.to(dev), out_big[1:1 + T])
+    assert torch.equal(out_big[1:1 + T].cpu(), torch.sum(x, dim=1))
+    assert bool((out_big[0] == 9.0).all()) and bool((out_big[T + 1] == 9.0).all())
+
+
 def test_moe_sum_strided_views_and_untouched_neighbours(ops, dev):
     """Input as a view with padded token and expert strides, output as a row slice of a larger
     tensor (how fused_experts passes out[begin:end]); everything outside the slice keeps its bytes."""
