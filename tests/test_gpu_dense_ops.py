@@ -238,6 +238,36 @@ def test_rope_shapes_bit_exact(ops, dev, T, nq, nkv, D, R, is_neox):
         assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("is_neox", [True, False])
+def test_rope_bf16_subnormal_range_and_signed_zeros(ops, dev, is_neox):
+    """The bf16 vector path forms each sum of two rounded products with the packed dot-product
+    instruction, which truncates its fp32 result instead of rounding it to nearest; that cannot
+    change the result once it is rounded to bf16.  Checked where it would show first: inputs
+    around 2^-121, so that many products and sums are subnormal.  Every non-zero output matches
+    the oracle bit for bit; an exactly zero output matches in value (the instruction returns +0
+    where the reference's subtraction returns -0)."""
+    g = gen(77)
+    T, nq, nkv, D = 64, 32, 8, 128
+    cache = cos_sin_cache(8192, D, THETA_LLAMA3, torch.bfloat16)
+    pos = hybrid_positions(T, 32, g)
+    q = (randn((T, nq * D), g, torch.float32) * 2.0 ** -121).to(torch.bfloat16)
+    k = (randn((T, nkv * D), g, torch.float32) * 2.0 ** -121).to(torch.bfloat16)
+    q[:, ::7] = 0.0
+    k[:, ::5] = -0.0
+    k[:, 1::5] = -0.0
+    wq, wk = q.clone(), k.clone()
+    c_oracle.rotary_embedding(pos, wq, wk, D, cache, is_neox)
+    gq, gk = q.to(dev), k.to(dev)
+    ops.pos_encoding_ops.rotary_embedding(pos.to(dev), gq, gk, D, cache.to(dev), is_neox)
+    subnormal = 0
+    for got, want in ((gq.cpu(), wq), (gk.cpu(), wk)):
+        assert torch.equal(got, want)                       # by value: -0 == +0
+        nz = want != 0
+        assert torch.equal(got.view(torch.int16)[nz], want.view(torch.int16)[nz])
+        subnormal += int(((want.float().abs() < 2.0 ** -126) & nz).sum())
+    assert subnormal > 1000, "inputs were meant to reach the subnormal range"
+
+
 def test_rope_position_zero_is_identity_and_norm_preserved(ops, dev):
     g = gen(8)
     T, nq, nkv, D = 256, 32, 8, 128
