@@ -141,10 +141,10 @@ int sarathi_topk_softmax(float* topk_weights, int32_t* topk_indices,
  * behaviour for them is undefined).
  *
  * `workspace` is optional device scratch of `workspace_bytes` bytes (4-byte
- * aligned, contents irrelevant on entry and exit).  Without it, or when it is
- * smaller than sarathi_moe_align_workspace_bytes() asks for, the sort runs in a
- * single workgroup, which is the fastest path up to ~16 K ids; with it, larger
- * inputs are spread over the whole GPU in three launches.  Results are
+ * aligned, contents irrelevant on entry and exit).  Up to 32 768 ids of at most 256 experts the
+ * sort is one launch of several independent workgroups and uses no scratch.  Beyond that, with a
+ * workspace of at least sarathi_moe_align_workspace_bytes() bytes, the input is spread over the
+ * whole GPU in three launches; without one the sort runs in a single workgroup.  Results are
  * identical either way.
  */
 int sarathi_moe_align_block_size(const void* topk_ids, int id_dtype, int64_t numel,
@@ -156,7 +156,7 @@ int sarathi_moe_align_block_size(const void* topk_ids, int id_dtype, int64_t num
 
 /*
  * Scratch bytes sarathi_moe_align_block_size can make use of for this input
- * size; 0 when the single-workgroup path will be taken anyway.  The reference
+ * size; 0 when a path without scratch will be taken anyway.  The reference
  * allocates a workspace in the same way for topk_softmax
  * (csrc/moe_topk_softmax_kernels.cu:486-492).
  */
@@ -208,9 +208,9 @@ int sarathi_grouped_topk(float* topk_weights, int32_t* topk_indices, const float
  * fused_topk -> moe_align_block_size (sarathi/model_executor/layers/fused_moe/fused_moe.py:346-373
  * and :151-204).  Outputs are bit-identical to the two separate calls.  `counter` is one uint32
  * of device memory that is zero before the first call; the call leaves it zero again.  Calls
- * that share a counter must not overlap (use one counter per stream).  With counter = NULL, with
- * an expert count that is not a power of two up to 256, or with more than 16384 ids, the two
- * stand-alone kernels are launched instead.
+ * that share a counter must not overlap (use one counter per stream).  The single launch is taken
+ * up to 1024 ids and a power-of-two expert count up to 16, where it is faster; with counter =
+ * NULL or any other shape the two stand-alone kernels are launched instead.
  */
 int sarathi_fused_topk_align(float* topk_weights, int32_t* topk_indices,
                              int32_t* token_expert_indices, const float* gating_output,

@@ -32,6 +32,30 @@ SK_DEV TileMatch match_expert(int e, bool valid, int nbits) {
   return m;
 }
 
+// Ids are fetched with raw buffer loads from a resource that covers the wave's part of the array:
+// positions past the end return 0 from the hardware range check and are discarded afterwards by
+// position, so no load sits under a per-lane condition.  (A plain load under one,
+// `i < numel ? ids[i] : -1`, compiles to a branch around the load with a wait for it right
+// behind -- the optimiser does the same to an unconditional load that feeds only one arm of a
+// select -- so a batch of such loads runs one after the other, 0.15 us each from L2, instead of
+// all being in flight together.)  COHERENT: the ids were written by other workgroups of the same
+// launch; the load is marked sc1 so that it does not hit in this compute unit's own cache.
+template <typename IdT, bool COHERENT = false> SK_DEV IdT buf_load_id(rsrc_t r, uint32_t byte_off) {
+  constexpr int kPolicy = COHERENT ? 16 : 0;
+  if constexpr (sizeof(IdT) == 1) return (IdT)__builtin_amdgcn_raw_buffer_load_b8(r, byte_off, 0, kPolicy);
+  else if constexpr (sizeof(IdT) == 2) return (IdT)__builtin_amdgcn_raw_buffer_load_b16(r, byte_off, 0, kPolicy);
+  else if constexpr (sizeof(IdT) == 4) return (IdT)__builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, kPolicy);
+  else {
+    const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(r, byte_off, 0, kPolicy);
+    return (IdT)(((uint64_t)v.y << 32) | v.x);
+  }
+}
+// Resource over ids[first, numel), at most 4 GiB - 1 of it (callers stay far below that).
+template <typename IdT> SK_DEV rsrc_t id_rsrc(const IdT* ids, int64_t first, int64_t numel) {
+  const int64_t left = first < numel ? (numel - first) * (int64_t)sizeof(IdT) : 0;
+  return make_rsrc(ids + (first < numel ? first : 0), left < 0xffffffffLL ? (uint32_t)left : 0xffffffffu);
+}
+
 // ids outside [0, E) become -1 (skipped); done in 64 bits so wide ids cannot wrap into range
 template <typename IdT> SK_DEV int checked_expert(IdT raw, int E) {
   const int64_t v = (int64_t)raw;
@@ -54,7 +78,7 @@ SK_DEV void align_single_workgroup(const IdT* __restrict__ ids, int64_t numel, i
   const int tid = threadIdx.x;
   const int nthr = blockDim.x;
   const int W = nthr >> 6;  // 16 or 8: a power of two
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be
   const int lane = tid & 63;
 
   for (int i = tid; i < W * E; i += nthr) cnt[i] = 0;
@@ -69,18 +93,14 @@ SK_DEV void align_single_workgroup(const IdT* __restrict__ ids, int64_t numel, i
   // small inputs: the wave's whole chunk stays in registers between the two passes
   const bool resident = tiles_per_wave <= kAlignBatch;
 
+  const rsrc_t rid = id_rsrc(ids, tile_lo << 6, numel);  // this wave's chunk
   auto load_batch = [&](int64_t t0, int (&e)[kAlignBatch]) {
 #pragma unroll
     for (int u = 0; u < kAlignBatch; ++u) {
       const int64_t i = ((t0 + u) << 6) + lane;
-      if constexpr (COHERENT) {
-        e[u] = (t0 + u < tile_hi && i < numel)
-                   ? checked_expert(__hip_atomic_load(ids + i, __ATOMIC_RELAXED,
-                                                      __HIP_MEMORY_SCOPE_AGENT), E)
-                   : -1;
-      } else {
-        e[u] = (t0 + u < tile_hi && i < numel) ? checked_expert(ids[i], E) : -1;
-      }
+      const IdT raw = buf_load_id<IdT, COHERENT>(
+          rid, (uint32_t)((((t0 + u - tile_lo) << 6) + lane) * (int64_t)sizeof(IdT)));
+      e[u] = (t0 + u < tile_hi && i < numel) ? checked_expert(raw, E) : -1;
     }
   };
   // cnt is indexed [e * W + wave]; only this wave touches its column, so plain LDS adds suffice

@@ -14,8 +14,13 @@
 // wave reaches its exit whatever the others do.  The counter must be zero on entry and is zero
 // again on exit; calls that share a counter must not overlap.
 //
-// Shapes the fused kernel does not cover (expert count not a power of two or above 256, more than
-// 16384 ids) take the two stand-alone launches; results are identical either way.
+// The one launch pays only while the sort is small: its last workgroup sorts alone, on one compute
+// unit, where the stand-alone moe_align_block_size spreads over several.  Measured on MI355X
+// (8 experts, top-2, launches issued back to back): 32 ids 5.7 us against 6.8 us for the two
+// launches, 1024 ids 6.7 against 6.7, 4096 ids 9.0 against 7.7, 8192 ids 12.5 against 8.9; with 64
+// experts and top-6 it loses from 384 ids on.  So the entry point runs the fused kernel up to
+// 1024 ids and 16 experts (a power of two) and the two stand-alone launches otherwise; results are
+// identical either way.
 #include "moe_align_body.h"
 #include "moe_topk_body.h"
 #include "launch.h"
@@ -23,7 +28,8 @@
 namespace sarathi_hip {
 
 constexpr int kFusedWaves = 16;
-constexpr int64_t kFusedMaxIds = 16384;
+constexpr int64_t kFusedMaxIds = 1024;
+constexpr int kFusedMaxExperts = 16;
 
 template <int E>
 __global__ __launch_bounds__(64 * kFusedWaves) void fused_topk_align_kernel(
@@ -105,7 +111,7 @@ extern "C" int sarathi_fused_topk_align(float* topk_weights, int32_t* topk_indic
     return SARATHI_ERR_INVALID_ARG;
   const int E = num_experts;
   const bool fusable = counter != nullptr && num_tokens > 0 && numel <= kFusedMaxIds &&
-                       (E & (E - 1)) == 0 && E <= 256 &&
+                       (E & (E - 1)) == 0 && E <= kFusedMaxExperts &&
                        (reinterpret_cast<uintptr_t>(gating_output) & (E < 4 ? E * 4 - 1 : 15)) == 0;
   if (!fusable) {
     // (zero tokens: topk_softmax is a no-op and the sort still writes num_tokens_post_pad = 0)

@@ -64,14 +64,14 @@ def pack_expert_weights(w: torch.Tensor, inplace: bool = False) -> PackedExpertW
     return PackedExpertWeights(tiles, (E, N, K))
 
 
-# fused_moe routes with the one-launch kernel (top-k + slot sort) up to this many (token, k) slots
-# and experts.  Measured on MI355X, launches issued back to back from Python, E = 8, top-2:
-#   tokens     16     256    1024   2304   4096
-#   two ops    7.3    7.6    8.6    11.0   13.4  us
-#   one launch 5.9    5.8    7.9    11.0   14.1  us
-# Small batches gain a launch; from a few thousand slots on the sorting workgroup's device-coherent
-# reads of the ids cost more than the launch saved (and at 64 experts x top-6 there is no gain).
-FUSED_ROUTING_MAX_SLOTS = 2048
+# fused_moe asks for routing and slot sort in one call (fused_topk_align) up to this many
+# (token, k) slots and experts; the op itself runs them as one launch up to 1024 slots and as the
+# two stand-alone kernels above that.  Measured on MI355X, launches issued back to back from
+# Python, E = 8, top-2:
+#   tokens      16     256    512    1024   2048   4096
+#   two ops     6.8    6.9    6.7    7.1    7.7    8.9   us
+#   one launch  5.7    6.1    6.7    7.3    9.0    12.5  us
+FUSED_ROUTING_MAX_SLOTS = 1024
 FUSED_ROUTING_MAX_EXPERTS = 16
 # silu_and_mul inside the gate/up GEMM's epilogue (same bits as the separate kernel)
 FUSE_SILU_AND_MUL = True

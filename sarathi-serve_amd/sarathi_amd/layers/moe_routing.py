@@ -60,8 +60,8 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int,
 
 def fused_topk_and_align(hidden_states: torch.Tensor, gating_output: torch.Tensor, topk: int,
                          renormalize: bool, block_size: int):
-    """``fused_topk`` followed by ``moe_align_block_size`` as ONE kernel launch (up to 16384
-    (token, k) slots and a power-of-two expert count up to 256; other shapes run the two kernels).
+    """``fused_topk`` followed by ``moe_align_block_size`` in one call: ONE kernel launch up to
+    1024 (token, k) slots and a power-of-two expert count up to 16; other shapes run the two kernels.
     Returns (topk_weights, topk_ids, sorted_token_ids, expert_ids, num_tokens_post_padded), the
     same tensors the two separate calls return."""
     assert hidden_states.shape[0] == gating_output.shape[0], "Number of tokens mismatch"

@@ -116,7 +116,7 @@ def test_topk_softmax_through_the_c_abi(lib, dev, T, E, k):
     torch.testing.assert_close(gw.cpu(), ww, atol=1e-6, rtol=0)
 
 
-@pytest.mark.parametrize("numel,E,B", [(8192, 8, 64), (50_000, 8, 64), (20_000, 200, 16)])
+@pytest.mark.parametrize("numel,E,B", [(8192, 8, 64), (50_000, 8, 64), (20_000, 300, 16), (20_000, 200, 16)])
 @pytest.mark.parametrize("with_workspace", [False, True])
 def test_moe_align_block_size_through_the_c_abi(lib, dev, numel, E, B, with_workspace):
     g = gen(104 + numel)
@@ -126,7 +126,8 @@ def test_moe_align_block_size_through_the_c_abi(lib, dev, numel, E, B, with_work
     idd = ids.to(dev)
     s, e, p = abi.align_buffers(numel, E, B, dev)
     need = lib.sarathi_moe_align_workspace_bytes(numel, E) if with_workspace else 0
-    assert (need > 0) == (with_workspace and numel > 16384)
+    # scratch is of use above 32 768 ids, or above 16 384 with more than 256 experts
+    assert (need > 0) == (with_workspace and (numel > 32768 or (numel > 16384 and E > 256)))
     scratch = torch.empty((need,), dtype=torch.uint8, device=dev) if need else None
     abi.check(lib, lib.sarathi_moe_align_block_size(
         abi.ptr(idd), abi.ID_DT[ids.dtype], numel, E, B, abi.ptr(s), s.numel(), abi.ptr(e),

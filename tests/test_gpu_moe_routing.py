@@ -136,7 +136,9 @@ def test_moe_align_reference_vectors(ops, dev):
                                      (1, 1, 8, 64), (7, 2, 8, 32), (63, 1, 4, 4), (64, 1, 4, 4),
                                      (65, 3, 16, 1), (1000, 6, 64, 16), (3000, 8, 256, 32),
                                      (500, 4, 1000, 8), (70000, 2, 8, 64), (16384, 4, 60, 128),
-                                     (8193, 2, 8, 64), (30000, 4, 1000, 8), (65536, 8, 256, 16)])
+                                     (8193, 2, 8, 64), (30000, 4, 1000, 8), (65536, 8, 256, 16),
+                                     (16000, 2, 8, 64), (16384, 2, 32, 16), (5461, 6, 64, 32),
+                                     (257, 1, 17, 4), (300, 1, 2, 1)])
 def test_moe_align_matches_oracle(ops, dev, T, k, E, B, filled):
     g = gen(T + E)
     ids = torch.randint(0, E, (T, k), generator=g, dtype=torch.int32)
@@ -243,14 +245,14 @@ def _separate(ops, dev, gating, k, renorm, E, B):
 
 
 @pytest.mark.parametrize("T,E,k,B,renorm", [
-    (4096, 8, 2, 64, True),        # Mixtral routing of the benchmark batch
-    (4096, 8, 2, 128, False),
+    (4096, 8, 2, 64, True),        # Mixtral routing of the benchmark batch: two launches
+    (512, 8, 2, 64, True),         # 1024 slots: the largest case that runs as ONE launch
+    (513, 8, 2, 128, False),       # one token too many: two launches, same results
     (1, 8, 2, 16, True),           # a single token: one workgroup, which is also the last one
     (17, 2, 1, 4, False),
-    (515, 64, 6, 32, True),        # several workgroups, ragged last row block
-    (2048, 256, 8, 16, False),     # 16384 slots: the largest fused case
-    (300, 16, 4, 64, True),
-    (2049, 256, 8, 16, True),      # one slot too many: two launches, same results
+    (170, 16, 6, 32, True),        # several workgroups, ragged last row block
+    (256, 16, 4, 64, True),
+    (100, 32, 4, 16, False),       # more than 16 experts: two launches
     (700, 60, 4, 32, False),       # expert count not a power of two: two launches
 ])
 def test_fused_topk_align_equals_separate_ops(ops, dev, T, E, k, B, renorm):
@@ -277,7 +279,7 @@ def test_fused_topk_align_equals_separate_ops(ops, dev, T, E, k, B, renorm):
 
 def test_fused_topk_align_against_oracle(ops, dev):
     """The one-launch path against the CPU oracle directly (not only against the other kernels)."""
-    T, E, k, B = 1000, 8, 2, 64
+    T, E, k, B = 500, 8, 2, 64
     gating = torch.randn((T, E), generator=gen(77), dtype=torch.float32)
     _assert_separated(gating, k)
     ww, wi, ws = _topk_oracle(gating, k)

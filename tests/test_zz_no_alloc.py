@@ -49,9 +49,9 @@ def _same(got, want, B):
 def test_static_scratch_entry_matches_workspace_entry_twice(dev):
     lib = abi.load()
     g = torch.Generator().manual_seed(41)
-    # both sizes take the three-launch path (above 16 384 ids), i.e. both use the scratch; the
-    # second call is smaller, so stale words of the first call's table lie beyond what it writes
-    cases = [(200_000, 64, 32, torch.int32), (40_000, 8, 64, torch.int64), (17_000, 5, 16, torch.int16)]
+    # all sizes take the three-launch path (above 32 768 ids), i.e. all use the scratch; every
+    # call is smaller than the one before, so stale words of the first call's table lie beyond what it writes
+    cases = [(200_000, 64, 32, torch.int32), (40_000, 8, 64, torch.int64), (36_000, 5, 16, torch.int16)]
     for numel, E, B, dt in cases:
         ids = torch.randint(0, E, (numel,), generator=g, dtype=torch.int32).to(dt)
         assert lib.sarathi_moe_align_workspace_bytes(numel, E) > 0
@@ -66,8 +66,8 @@ def test_static_scratch_entry_matches_workspace_entry_twice(dev):
 def test_static_scratch_entry_small_inputs_and_limit(dev):
     lib = abi.load()
     g = torch.Generator().manual_seed(42)
-    # at or below 16 384 ids the single-workgroup path runs: no scratch at all
-    for numel, E, B in [(8192, 8, 64), (1, 8, 4), (0, 8, 4)]:
+    # small inputs take the one-launch or single-workgroup kernels: no scratch at all
+    for numel, E, B in [(8192, 8, 64), (20_000, 64, 16), (1, 8, 4), (0, 8, 4)]:
         ids = torch.randint(0, E, (numel,), generator=g, dtype=torch.int32)
         got = _run(lib, True, ids.to(dev), E, B, 1)
         _same(got, _oracle(ids, E, B), B)
