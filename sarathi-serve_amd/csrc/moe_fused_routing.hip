@@ -52,7 +52,11 @@ __global__ __launch_bounds__(64 * kFusedWaves) void fused_topk_align_kernel(
   // acknowledgement, which vmcnt counts, comes back once they are where every compute unit reads
   // coherently.  Every wave waits for its own stores here; the barrier that follows then tells
   // thread 0 that all ids of this workgroup are visible before it bumps the counter.  (The
-  // barrier alone does not: its workgroup-scope fence does not wait for global stores.)
+  // barrier alone does not: its workgroup-scope fence does not wait for global stores.)  The
+  // textbook form -- plain stores, an agent-scope acquire-release fetch-add on the counter, plain
+  // loads in the sorting workgroup -- is also correct and was measured: 5.4 / 6.0 / 6.7 / 7.3 us
+  // at 16 / 64 / 256 / 512 tokens (8 experts, top-2) against 5.5 / 5.8 / 6.2 / 7.1 us for this
+  // form; its release writes back and its acquire invalidates whole caches.
   wait_vmcnt<0>();
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -66,7 +70,6 @@ __global__ __launch_bounds__(64 * kFusedWaves) void fused_topk_align_kernel(
   align_single_workgroup<int32_t, true>(indices, num_tokens * k, E, B, nbits, sorted, sorted_len,
                                   expert_ids, expert_ids_len, post_pad, fill_pad, cnt, tot, cumsum);
 }
-
 template <int E>
 static void launch_fused(float* w, int32_t* idx, int32_t* src, const float* g, int64_t T, int k,
                          int renorm, int B, int32_t* sorted, int64_t sorted_len,
