@@ -6,16 +6,95 @@
 // append_paged_kv_cache with kv_layout="NHD".  The rotary-embedding + append fusion lives next to
 // the rotary kernel (rope.hip); this file holds the plain copy.
 //
-// append: a workgroup is one wave that moves 64 consecutive 16-byte pieces of one token's key row
-// or value row into the token's cache entry.  Workgroup ids run over the key pieces, then the value
-// pieces, then the tokens, so the waves in flight read the source linearly.  Source rows are read
-// with the streaming policy (they are not needed again), cache entries are written with the
-// default policy (attention reads them next).
+// append: a workgroup is one wave that moves the key row and the value row of one to four
+// consecutive tokens (rows of up to 4 KiB, every lane 16 bytes of up to four 1 KiB pieces).  The
+// index loads of all its tokens go out first, then all the row loads, and only then are the cache
+// entries resolved and written: the dependent page-table lookups run under the row loads instead
+// of in front of them.  Source rows are read with the streaming policy (they are not needed
+// again), cache entries are written with the default policy (attention reads them next).  Rows
+// longer than 4 KiB go through the older kernel of one wave per 1 KiB piece.
 #include "kv_dest.h"
 #include "launch.h"
 
 namespace sarathi_hip {
 
+// PPL pieces of 1 KiB per row (one 16-byte load per lane each), TPW tokens per wave; SLOTS says
+// whether a slot mapping is given (a kernel of its own each way keeps the order below free of
+// branches).  What the row loads need comes first in the argument list, where the kernel
+// arguments are preloaded into registers; the cache geometry is fetched under the row loads.
+// Tokens past the end of the batch get empty buffer resources: their loads return nothing and
+// their stores are dropped.
+template <int PPL, int TPW, bool SLOTS>
+__global__ __launch_bounds__(64) void kv_append_tok_kernel(
+    const void* __restrict__ key, const void* __restrict__ value, int64_t k_stride_bytes,
+    int64_t v_stride_bytes, uint32_t row_bytes, uint32_t nnz, const int32_t* __restrict__ index_a,
+    const int32_t* __restrict__ index_b, KvDest d) {
+  const uint32_t tok0 = blockIdx.x * TPW;
+  const uint32_t off = threadIdx.x * 16u;
+  KvEntryKey keys[TPW];
+  u32x4 kk[TPW][PPL], vv[TPW][PPL];
+  uint32_t recs[TPW];
+#pragma unroll
+  for (int t = 0; t < TPW; ++t) {
+    const bool live = tok0 + t < nnz;
+    const uint32_t tok = live ? tok0 + t : nnz - 1;
+    recs[t] = live ? row_bytes : 0u;
+    keys[t].a = index_a[tok];  // slot, or request
+    keys[t].b = SLOTS ? 0 : index_b[tok];
+  }
+#pragma unroll
+  for (int t = 0; t < TPW; ++t) {
+    const rsrc_t rk = make_rsrc(
+        reinterpret_cast<const char*>(key) + (int64_t)(tok0 + t) * k_stride_bytes, recs[t]);
+    const rsrc_t rv = make_rsrc(
+        reinterpret_cast<const char*>(value) + (int64_t)(tok0 + t) * v_stride_bytes, recs[t]);
+#pragma unroll
+    for (int p = 0; p < PPL; ++p) kk[t][p] = buf_load16<kStreamLoad>(rk, off + p * 1024u);
+#pragma unroll
+    for (int p = 0; p < PPL; ++p) vv[t][p] = buf_load16<kStreamLoad>(rv, off + p * 1024u);
+  }
+  __builtin_amdgcn_sched_barrier(0);  // every load is issued before anything waits
+#pragma unroll
+  for (int t = 0; t < TPW; ++t) {
+    const int64_t e = kv_entry_resolve<SLOTS>(d, keys[t]);
+    const rsrc_t dk = make_rsrc(reinterpret_cast<char*>(d.k_cache) + e, recs[t]);
+    const rsrc_t dv = make_rsrc(reinterpret_cast<char*>(d.v_cache) + e, recs[t]);
+#pragma unroll
+    for (int p = 0; p < PPL; ++p) buf_store16<kKvStore>(dk, off + p * 1024u, kk[t][p]);
+#pragma unroll
+    for (int p = 0; p < PPL; ++p) buf_store16<kKvStore>(dv, off + p * 1024u, vv[t][p]);
+  }
+}
+
+template <int PPL>
+static void launch_kv_tok(hipStream_t st, const void* key, const void* value, int64_t ksb,
+                          int64_t vsb, uint32_t row_bytes, const KvDest& d) {
+  const int tpw = pick_rows_per_workgroup(d.nnz, 4 / PPL);
+  const unsigned grid = (unsigned)((d.nnz + tpw - 1) / tpw);
+  const uint32_t nnz = (uint32_t)d.nnz;
+#define SARATHI_KV_TOK(T)                                                                        \
+  do {                                                                                           \
+    if (d.slot_mapping)                                                                          \
+      hipLaunchKernelGGL((kv_append_tok_kernel<PPL, T, true>), dim3(grid), dim3(64), 0, st, key, \
+                         value, ksb, vsb, row_bytes, nnz, d.slot_mapping, nullptr, d);           \
+    else                                                                                         \
+      hipLaunchKernelGGL((kv_append_tok_kernel<PPL, T, false>), dim3(grid), dim3(64), 0, st,     \
+                         key, value, ksb, vsb, row_bytes, nnz, d.batch_indices, d.positions, d); \
+  } while (0)
+  if constexpr (PPL == 1) {
+    if (tpw == 4) { SARATHI_KV_TOK(4); return; }
+    if (tpw == 3) { SARATHI_KV_TOK(3); return; }
+  }
+  if constexpr (PPL <= 2) {
+    if (tpw == 2) { SARATHI_KV_TOK(2); return; }
+  }
+  SARATHI_KV_TOK(1);
+#undef SARATHI_KV_TOK
+}
+
+// Rows of any length: a workgroup is one wave that moves 64 consecutive 16-byte pieces of one
+// token's key row or value row.  Workgroup ids run over the key pieces, then the value pieces,
+// then the tokens.
 __global__ __launch_bounds__(64) void kv_append_seg_kernel(
     const void* __restrict__ key, const void* __restrict__ value, int64_t k_stride_bytes,
     int64_t v_stride_bytes, uint32_t row_bytes, uint32_t blocks_per_row, KvDest d) {
@@ -125,6 +204,12 @@ extern "C" int sarathi_append_paged_kv_cache(
   if (!vec_ok) {
     hipLaunchKernelGGL(kv_append_generic_kernel, dim3((unsigned)nnz), dim3(256), 0, st, append_key,
                        append_value, ksb, vsb, row_bytes, d);
+    return launch_status();
+  }
+  if (row_bytes <= 4096) {
+    if (row_bytes <= 1024) launch_kv_tok<1>(st, append_key, append_value, ksb, vsb, row_bytes, d);
+    else if (row_bytes <= 2048) launch_kv_tok<2>(st, append_key, append_value, ksb, vsb, row_bytes, d);
+    else launch_kv_tok<4>(st, append_key, append_value, ksb, vsb, row_bytes, d);
     return launch_status();
   }
   const uint32_t bpr = (row_bytes / 16 + 63) / 64;

@@ -55,8 +55,10 @@ SK_DEV KvEntryKey kv_entry_key(const KvDest& d, int64_t tok) {
   }
   return k;
 }
+// SLOTS: whether k.a is a slot (known at compile time where a kernel is specialised on it).
+template <bool SLOTS>
 SK_DEV int64_t kv_entry_resolve(const KvDest& d, KvEntryKey k) {
-  if (d.slot_mapping != nullptr) {
+  if (SLOTS) {
     const uint32_t slot = (uint32_t)k.a;
     const uint32_t page = slot / (uint32_t)d.page_size;
     const uint32_t entry = slot - page * (uint32_t)d.page_size;
@@ -67,6 +69,9 @@ SK_DEV int64_t kv_entry_resolve(const KvDest& d, KvEntryKey k) {
   const uint32_t entry = pos - pg * (uint32_t)d.page_size;
   const int64_t page = d.kv_indices[(int64_t)d.kv_indptr[k.a] + pg];
   return page * d.page_stride_bytes + (int64_t)entry * d.entry_stride_bytes;
+}
+SK_DEV int64_t kv_entry_resolve(const KvDest& d, KvEntryKey k) {
+  return d.slot_mapping != nullptr ? kv_entry_resolve<true>(d, k) : kv_entry_resolve<false>(d, k);
 }
 SK_DEV int64_t kv_entry_offset(const KvDest& d, int64_t tok) {
   return kv_entry_resolve(d, kv_entry_key(d, tok));

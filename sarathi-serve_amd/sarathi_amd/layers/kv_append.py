@@ -5,7 +5,11 @@ sarathi/model_executor/attention/flashinfer_attention_wrapper.py:84-229).
 A batch is prefill chunks first, then one decode token per running request.  For every request
 the page table prefix in use, the fill of its last page and the start of its tokens in the
 flattened batch are collected into the four int32 vectors the append needs; the two derived
-vectors (request index and kv position of every token) come from the device helpers.
+vectors (request index and kv position of every token) come from the device helpers, and so does
+the slot of every token (page * block_size + entry), which is the same for all layers of the
+model: it is computed once here and every append of the batch (``AppendMetadata.append``,
+``AppendMetadata.rotary_embedding_append``) passes it on, so that the per-layer kernels do one
+index load per token instead of three dependent ones.
 """
 from dataclasses import dataclass
 from typing import List, Sequence
@@ -37,6 +41,26 @@ class AppendMetadata:
     slot_mapping: torch.Tensor              # [num_total_tokens] page * block_size + entry
     num_prefill_tokens: int
     num_total_tokens: int
+
+    def append(self, key: torch.Tensor, value: torch.Tensor, kv_cache, kv_layout: str = "NHD") -> None:
+        """The append of FlashinferAttentionWrapper.forward
+        (sarathi/model_executor/attention/flashinfer_attention_wrapper.py:262-273) for this batch:
+        ``key`` / ``value`` ``[num_total_tokens, num_kv_heads, head_size]`` go into ``kv_cache``."""
+        kv_cache_ops.append_paged_kv_cache(
+            key, value, self.append_batch_indices, self.append_positions, kv_cache,
+            self.append_kv_page_indices, self.append_kv_page_indptr, self.append_kv_last_page_len,
+            kv_layout=kv_layout, slot_mapping=self.slot_mapping)
+
+    def rotary_embedding_append(self, positions: torch.Tensor, query: torch.Tensor,
+                                key: torch.Tensor, value: torch.Tensor, head_size: int,
+                                cos_sin_cache: torch.Tensor, is_neox: bool, kv_cache,
+                                write_key: bool = False, kv_layout: str = "NHD") -> None:
+        """Rotary embedding of ``query`` / ``key`` and the append above in one launch."""
+        kv_cache_ops.rotary_embedding_append_paged_kv(
+            positions, query, key, value, head_size, cos_sin_cache, is_neox,
+            self.append_batch_indices, self.append_positions, kv_cache,
+            self.append_kv_page_indices, self.append_kv_page_indptr, self.num_total_tokens,
+            write_key, kv_layout, slot_mapping=self.slot_mapping)
 
 
 def build_append_metadata(seqs: Sequence[SequenceSlice], block_size: int,

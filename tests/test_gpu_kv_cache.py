@@ -105,6 +105,42 @@ def test_append_matches_oracle_bitwise(ops, dev, dtype, page_size, before, new, 
     assert np.array_equal(_bits(got2.cpu()), want)
 
 
+@pytest.mark.parametrize("nnz,heads,head_size,dtype", [
+    (3001, 4, 64, torch.bfloat16),    # 512-byte rows: several tokens per wave, ragged last wave
+    (2050, 1, 8, torch.bfloat16),     # one 16-byte piece per row
+    (3003, 8, 96, torch.float16),     # 1.5 KiB rows: two pieces per lane, the second half empty
+    (1031, 8, 96, torch.float32),     # 3 KiB rows
+    (600, 8, 128, torch.float32),     # exactly 4 KiB
+    (517, 16, 160, torch.bfloat16),   # 5 KiB rows: one wave per KiB piece
+])
+@pytest.mark.parametrize("use_slots", [False, True])
+def test_append_every_row_length_class(ops, dev, nnz, heads, head_size, dtype, use_slots):
+    """One request whose tokens land on shuffled pages; checked by indexing the cache with the
+    slots, which is the definition of the layout (entry e of page p holds slot p * page_size + e)."""
+    page_size = 16
+    pages = (nnz + page_size - 1) // page_size
+    g = gen(nnz)
+    table = torch.randperm(pages + 5, generator=g)[:pages].to(torch.int32)
+    k = randn((nnz, heads, head_size), g, dtype).to(dev)
+    v = randn((nnz, heads, head_size), g, dtype).to(dev)
+    cache = randn((pages + 5, 2, page_size, heads, head_size), g, dtype).to(dev)
+    before = cache.clone()
+    b = torch.zeros(nnz, dtype=torch.int32, device=dev)
+    pos = torch.arange(nnz, dtype=torch.int32, device=dev)
+    indptr = torch.tensor([0, pages], dtype=torch.int32, device=dev)
+    slots = (table.long()[torch.arange(nnz) // page_size] * page_size
+             + torch.arange(nnz) % page_size).to(dev)
+    ops.kv_cache_ops.append_paged_kv_cache(
+        k, v, b, pos, cache, table.to(dev), indptr,
+        slot_mapping=slots.to(torch.int32) if use_slots else None)
+    flat = cache.permute(0, 2, 1, 3, 4).reshape(-1, 2, heads, head_size)   # [slot, k/v, heads, D]
+    assert torch.equal(flat[slots, 0], k) and torch.equal(flat[slots, 1], v)
+    untouched = torch.ones(flat.shape[0], dtype=torch.bool, device=dev)
+    untouched[slots] = False
+    assert torch.equal(flat[untouched],
+                       before.permute(0, 2, 1, 3, 4).reshape(flat.shape)[untouched])
+
+
 def _rope_then_append(positions, q, k, v, head_size, table, is_neox, b, pos, cache, kv_indices,
                       kv_indptr, n):
     """The reference sequence on the CPU: rotary_embedding in place, then append the first n rows."""
@@ -201,6 +237,7 @@ def test_hybrid_batch_full_size_round_trip(ops, dev):
     cache = torch.zeros((len(perm), 2, page_size, nkv, D), dtype=torch.bfloat16, device=dev)
     q, k, v = qkv.split([nq * D, nkv * D, nkv * D], dim=-1)
     ref = qkv.clone()
+    qkv_before = qkv.clone()
     rq, rk, rv = ref.split([nq * D, nkv * D, nkv * D], dim=-1)
     ops.pos_encoding_ops.rotary_embedding(positions, rq, rk, D, table, True)
     ops.kv_cache_ops.rotary_embedding_append_paged_kv(
@@ -214,6 +251,14 @@ def test_hybrid_batch_full_size_round_trip(ops, dev):
                                            meta.append_kv_page_indices, meta.append_kv_page_indptr,
                                            meta.append_kv_last_page_len)
     assert torch.equal(cache, cache2)
+    # the batch's own methods (slot mapping computed once per batch) give the same bytes again
+    cache3, cache4 = torch.zeros_like(cache), torch.zeros_like(cache)
+    meta.append(rk.reshape(T, nkv, D), rv.reshape(T, nkv, D), cache3)
+    qkv2 = ref.clone()
+    qkv2.copy_(qkv_before)
+    q2, k2, v2 = qkv2.split([nq * D, nkv * D, nkv * D], dim=-1)
+    meta.rotary_embedding_append(positions, q2, k2, v2, D, table, True, cache4)
+    assert torch.equal(cache, cache3) and torch.equal(cache, cache4) and torch.equal(q2, rq)
     # read back through the page table
     qo = meta.append_qo_indptr.cpu().tolist()
     indptr = meta.append_kv_page_indptr.cpu().tolist()
