@@ -3,9 +3,11 @@ sarathi/model_executor/layers/fused_moe/fused_moe.py:207-260 and :411-622).
 
 ``fused_moe`` = top-k routing -> slot sort (moe_align_block_size) -> grouped GEMM with w1 ->
 silu_and_mul -> grouped GEMM with w2 (times the routing weight) -> sum over the k slots of a token.
-The two GEMMs are one hand-written MFMA kernel (csrc/moe_gemm.hip) instead of the reference's
-Triton kernel; there are no tuning JSON files, the slot-block size is picked from the batch size.
-fp8 weights / scales are not supported.
+The two GEMMs are hand-written MFMA kernels (csrc/moe_gemm.hip, csrc/moe_gemm_wide.hip) instead of
+the reference's Triton kernel.  Their only free parameter is the slot-block size, which comes from
+the tuned tables under ``configs/`` (the reference's JSON format, written by tune_fused_moe.py)
+when one matches (E, N, device, weight layout), else from ``get_default_config``.
+float16 and bfloat16 only: float32 activations / weights and fp8 weights / scales raise.
 """
 import functools
 import json
@@ -186,7 +188,11 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
     assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
     assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
     assert w1.is_contiguous() and w2.is_contiguous(), "Expert weights must be contiguous"
-    assert hidden_states.dtype in (torch.float16, torch.bfloat16)
+    if hidden_states.dtype not in (torch.float16, torch.bfloat16) or w1.dtype != hidden_states.dtype \
+            or w2.dtype != hidden_states.dtype:
+        raise TypeError("fused_experts runs on the float16 / bfloat16 matrix-core kernels only: got "
+                        f"hidden_states {hidden_states.dtype}, w1 {w1.dtype}, w2 {w2.dtype} (the "
+                        "reference's float32 path has no counterpart here; cast the layer)")
     assert w1_scale is None and w2_scale is None and a1_scale is None and a2_scale is None, \
         "fp8 scales are not supported"
     num_tokens, K = hidden_states.shape

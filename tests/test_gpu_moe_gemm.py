@@ -231,9 +231,29 @@ def test_tuned_config_lookup_and_override(ops, dev):
     rm = layers.get_moe_configs(8, 14336, None, packed=False)      # table for row-major weights
     assert rm is not None and rm[4096]["BLOCK_SIZE_M"] == 256
     assert layers.try_get_optimal_moe_config(w1_shape, w2_shape, 2, 4000, packed=False) == rm[4096]
+    # every Mixtral per-rank shape the reference ships a bf16 table for (its configs/ folder:
+    # E=8 with N = 14336, 7168, 3584, 1792) has one here, for both weight layouts
+    for n in (14336, 7168, 3584, 1792):
+        for packed in (True, False):
+            t = layers.get_moe_configs(8, n, None, packed=packed)
+            assert t is not None and {1, 64, 4096} <= set(t), (n, packed)
+            assert all(c["BLOCK_SIZE_M"] in (32, 64, 128, 256) for c in t.values())
     assert layers.get_moe_configs(7, 1234, None) is None
     assert layers.try_get_optimal_moe_config((7, 2468, 64), (7, 64, 1234), 2, 512) == \
         layers.get_default_config(512, 7, 1234, 64, 2)
+
+
+def test_fused_experts_rejects_float32(ops, dev):
+    """The reference's Triton kernel also takes float32; the matrix-core kernels here do not, and
+    say so instead of failing inside the launcher."""
+    from sarathi_amd import layers
+    x = torch.zeros((4, 64), device=dev)
+    w1, w2 = torch.zeros((2, 32, 64), device=dev), torch.zeros((2, 64, 16), device=dev)
+    tw, ti = torch.ones((4, 1), device=dev), torch.zeros((4, 1), dtype=torch.int32, device=dev)
+    with pytest.raises(TypeError, match="float16 / bfloat16"):
+        layers.fused_experts(x, w1, w2, tw, ti)
+    with pytest.raises(TypeError, match="float16 / bfloat16"):
+        layers.fused_experts(x.half(), w1.half(), w2, tw, ti)
 
 
 @pytest.mark.parametrize("grouped", [False, True])
