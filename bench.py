@@ -138,6 +138,10 @@ def main():
                     help="moe section: constant = every activation and weight holds the same value "
                          "(far fewer bits toggle per operation: shows how much of the gap to the "
                          "nominal MFMA peak is the clock the chip sustains under switching power)")
+    ap.add_argument("--moe-routing", choices=["random", "balanced"], default="random",
+                    help="moe section: random = N(0,1) router logits (experts get unequal shares, "
+                         "as in a real batch); balanced = every expert gets exactly tokens * top_k / "
+                         "experts slots (no partly filled slot blocks): shows what the imbalance costs")
     ap.add_argument("--moe-block-m", type=int, default=0,
                     help="moe section: slot-block size of the grouped GEMMs (0 = the library's choice)")
     args = ap.parse_args()
@@ -513,6 +517,15 @@ def main():
             return {"ms": round(ms, 4), "TFLOPs": round(flop / ms * 1e-9, 1),
                     "frac_of_mfma_peak": round(flop / ms * 1e-9 / MFMA_PEAK_TFLOPS, 4)}
 
+        def router_logits(Tn):
+            if args.moe_routing == "random":
+                return torch.randn((Tn, E), device=dev, dtype=torch.float32)
+            t = torch.arange(Tn, device=dev)
+            lg = torch.zeros((Tn, E), device=dev, dtype=torch.float32)
+            for j in range(k):                      # token t -> experts (k t + j) mod E
+                lg[t, (k * t + j) % E] = float(k - j)
+            return lg
+
         w1 = (torch.randn((E, 2 * I, Hm), device=dev, dtype=torch.float32) * Hm ** -0.5).to(bf16)
         w2 = (torch.randn((E, Hm, I), device=dev, dtype=torch.float32) * I ** -0.5).to(bf16)
         if args.moe_data == "constant":
@@ -523,7 +536,7 @@ def main():
             x = torch.randn((Tn, Hm), device=dev, dtype=torch.float32).to(bf16)
             if args.moe_data == "constant":
                 x.fill_(0.0078125)
-            logits = torch.randn((Tn, E), device=dev, dtype=torch.float32)
+            logits = router_logits(Tn)
             ms = timeit_ms(lambda: layers.fused_moe(x, w1, w2, logits, k, True))
             row = tflops(2.0 * Tn * k * 3 * I * Hm, ms)
             row["weight_stream_TBps"] = round((E * 3 * I * Hm * 2) / ms * 1e-9, 2)
@@ -533,7 +546,7 @@ def main():
         x = torch.randn((Tn, Hm), device=dev, dtype=torch.float32).to(bf16)
         if args.moe_data == "constant":
             x.fill_(0.0078125)
-        logits = torch.randn((Tn, E), device=dev, dtype=torch.float32)
+        logits = router_logits(Tn)
         tw_m, ti_m = layers.fused_topk(x, logits, k, True)
         c1 = torch.empty((Tn, k, 2 * I), device=dev, dtype=bf16)
         c2 = torch.empty((Tn * k, I), device=dev, dtype=bf16)
@@ -572,8 +585,8 @@ def main():
         torch.cuda.empty_cache()
         out["moe_layer"] = {
             "shape": "Mixtral-8x7B MoE layer: 8 experts, top-2, hidden 4096, intermediate 14336, "
-                     "bf16, %s data, back-to-back launches (weights warm in L2/MALL as far as "
-                     "they fit)" % args.moe_data,
+                     "bf16, %s data, %s routing, back-to-back launches (weights warm in L2/MALL "
+                     "as far as they fit)" % (args.moe_data, args.moe_routing),
             "peak": "2500 TFLOP/s dense bf16 MFMA; 8 TB/s HBM",
             "fused_moe_forward_row_major": forward, "at_4096_tokens": gemms}
 
