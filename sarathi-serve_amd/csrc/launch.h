@@ -20,14 +20,8 @@ static inline int launch_status() {
   return hipGetLastError() == hipSuccess ? SARATHI_OK : SARATHI_ERR_LAUNCH;
 }
 
-// Rows per workgroup for the kernels that put R consecutive rows into one one-wave workgroup
-// (fused_add_rms_norm, moe_sum).  Workgroups are dealt to the compute units in turn, so
-// the launch lasts as long as the busiest unit: ceil(workgroups / units) * R rows.  Take the
-// largest R (fewest weight fetches, fewest workgroups) among those with the shortest busiest
-// unit, but keep one row per workgroup while that leaves fewer than two workgroups per unit
-// (small batches need the parallelism more).  Measured at 2304 rows of 4096 bf16: R = 3 (768
-// workgroups, 3 per unit) 12.4 us, R = 2 (1152, i.e. 4.5 per unit) 15.6 us, R = 1 13.8 us.
-static inline int pick_rows_per_workgroup(int64_t rows, int max_rows_per_wg) {
+// Compute units of the current device (looked up once; 256 when the query fails).
+static inline int compute_units() {
   static const int units = [] {
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
@@ -38,6 +32,18 @@ static inline int pick_rows_per_workgroup(int64_t rows, int max_rows_per_wg) {
     }
     return n;
   }();
+  return units;
+}
+
+// Rows per workgroup for the kernels that put R consecutive rows into one one-wave workgroup
+// (fused_add_rms_norm, moe_sum).  Workgroups are dealt to the compute units in turn, so
+// the launch lasts as long as the busiest unit: ceil(workgroups / units) * R rows.  Take the
+// largest R (fewest weight fetches, fewest workgroups) among those with the shortest busiest
+// unit, but keep one row per workgroup while that leaves fewer than two workgroups per unit
+// (small batches need the parallelism more).  Measured at 2304 rows of 4096 bf16: R = 3 (768
+// workgroups, 3 per unit) 12.4 us, R = 2 (1152, i.e. 4.5 per unit) 15.6 us, R = 1 13.8 us.
+static inline int pick_rows_per_workgroup(int64_t rows, int max_rows_per_wg) {
+  const int units = compute_units();
   int best = 1;
   int64_t best_cost = (rows + units - 1) / units;
   for (int r = 2; r <= max_rows_per_wg; ++r) {
