@@ -231,12 +231,14 @@ def test_tuned_config_lookup_and_override(ops, dev):
     rm = layers.get_moe_configs(8, 14336, None, packed=False)      # table for row-major weights
     assert rm is not None and rm[4096]["BLOCK_SIZE_M"] == 256
     assert layers.try_get_optimal_moe_config(w1_shape, w2_shape, 2, 4000, packed=False) == rm[4096]
-    # every Mixtral per-rank shape the reference ships a bf16 table for (its configs/ folder:
-    # E=8 with N = 14336, 7168, 3584, 1792) has one here, for both weight layouts
-    for n in (14336, 7168, 3584, 1792):
+    # every (E, N) the reference ships a 16-bit table for (its configs/ folder) has one here, for
+    # both weight layouts
+    shapes = [(8, n) for n in (14336, 8192, 7168, 4096, 3584, 2048, 1792)] + \
+             [(16, 2688), (16, 1344), (64, 1280), (64, 640)]
+    for e, n in shapes:
         for packed in (True, False):
-            t = layers.get_moe_configs(8, n, None, packed=packed)
-            assert t is not None and {1, 64, 4096} <= set(t), (n, packed)
+            t = layers.get_moe_configs(e, n, None, packed=packed)
+            assert t is not None and {1, 64, 4096} <= set(t), (e, n, packed)
             assert all(c["BLOCK_SIZE_M"] in (32, 64, 128, 256) for c in t.values())
     assert layers.get_moe_configs(7, 1234, None) is None
     assert layers.try_get_optimal_moe_config((7, 2468, 64), (7, 64, 1234), 2, 512) == \
