@@ -99,7 +99,7 @@ __global__ __launch_bounds__(64 * kFewWaves) void moe_align_few_experts_kernel(
   __shared__ uint32_t red[kFewWaves][2][ACCS * 2];   // [wave][all / before][packed halves]
   __shared__ int32_t own[kFewWaves][EMAX];           // ids of expert e in wave w's own tile
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and the compiler knows it
   const int tiles_total = (int)((numel + 63) >> 6);
   const int wg_first = (int)blockIdx.x * kFewWaves;  // first own tile of the workgroup
   const int my_tile = wg_first + wave;               // the wave's own tile

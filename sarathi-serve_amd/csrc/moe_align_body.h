@@ -78,7 +78,7 @@ SK_DEV void align_single_workgroup(const IdT* __restrict__ ids, int64_t numel, i
   const int tid = threadIdx.x;
   const int nthr = blockDim.x;
   const int W = nthr >> 6;  // 16 or 8: a power of two
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and the compiler knows it
   const int lane = tid & 63;
 
   for (int i = tid; i < W * E; i += nthr) cnt[i] = 0;
