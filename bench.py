@@ -453,7 +453,7 @@ def main():
             rows = {}
             wn = dev_randn((Hn,))
             posn = hybrid_positions(Tn, Tn - Tn // 9, gen(4), prefill_start=4096,
-                                    max_pos=8192).to(dev) if "rotary_embedding" in which else None
+                                    max_pos=8192).to(dev) if any("rotary" in w for w in which) else None
             plan = {
                 "fused_add_rms_norm": (4 * Tn * Hn * BF16 + Hn * BF16,
                                        lambda: (dev_randn((Tn, Hn)), dev_randn((Tn, Hn))),
@@ -470,6 +470,19 @@ def main():
                                  lambda: (dev_randn((Tn, 2 * dff)),
                                           torch.empty((Tn, dff), dtype=bf16, device=dev)),
                                  lambda a: ACT.silu_and_mul(a[1], a[0])),
+                "gelu_new": (2 * Tn * dff * BF16,
+                             lambda: (dev_randn((Tn, dff)),
+                                      torch.empty((Tn, dff), dtype=bf16, device=dev)),
+                             lambda a: ACT.gelu_new(a[1], a[0])),
+                "gelu_fast": (2 * Tn * dff * BF16,
+                              lambda: (dev_randn((Tn, dff)),
+                                       torch.empty((Tn, dff), dtype=bf16, device=dev)),
+                              lambda a: ACT.gelu_fast(a[1], a[0])),
+                "rotary_embedding (GPT-J layout)": (
+                    2 * Tn * (nq + nkv) * D * BF16 + Tn * 8 + Tn * D * BF16,
+                    lambda: dev_randn((Tn, (nq + 2 * nkv) * D)),
+                    lambda a: ROPE.rotary_embedding(
+                        posn, *a.split([nq * D, nkv * D, nkv * D], dim=-1)[:2], D, cache_dev, False)),
             }
             for name in which:
                 nbytes, make, fn = plan[name]
@@ -483,6 +496,10 @@ def main():
             return rows
 
         other_configs = {
+            "rest of the module surface at the Llama-3-8B batch, T=2304: gelu_new / gelu_fast "
+            "[2304, 14336], rotary_embedding with interleaved (GPT-J) pairs":
+                measure_shape(T, H, NQ, NKV, DFF,
+                              ["gelu_new", "gelu_fast", "rotary_embedding (GPT-J layout)"]),
             "fused_add_rms_norm [512, 4096] (CPU-sized case)":
                 measure_shape(512, 4096, 32, 8, 14336, ["fused_add_rms_norm"]),
             "Llama-3-70B widths, T=4608: norm [4608, 8192], rope q[4608, 8192] k[4608, 1024], "

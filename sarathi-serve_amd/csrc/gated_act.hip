@@ -25,10 +25,10 @@ namespace sarathi_hip {
 constexpr int kActBlock = 256;   // element-wise fallback kernels
 constexpr int kRowSeg = 64;      // lanes per workgroup of the streaming kernels
 
-// tanh(u) = 1 - 2 / (1 + e^{2u}); the clamp keeps e^{2u} finite
+// tanh(u) = 1 - 2 / (1 + e^{2u}).  No clamp is needed: for large u the exponential is +inf, whose
+// reciprocal is 0 (result 1); for very negative u it is 0 (result -1); NaN passes through.
 SK_DEV float tanh_f32(float u) {
-  float c = u < -15.f ? -15.f : (u > 15.f ? 15.f : u);  // NaN passes through
-  float e = __builtin_amdgcn_exp2f(c * 2.8853900817779268f);
+  float e = __builtin_amdgcn_exp2f(u * 2.8853900817779268f);
   return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
@@ -103,23 +103,34 @@ static int launch_silu(void* out, const void* in, int64_t T, int64_t d, int64_t 
 
 // ---- gelu_new / gelu_fast ----------------------------------------------------
 
-template <int DT> SK_DEV float gelu_new_elem(float x) {
-  float x3 = rnd<DT>(rnd<DT>(x * x) * x);
-  float a = rnd<DT>(0.044715f * x3);
-  float b = rnd<DT>(x + a);
-  float c = rnd<DT>(0.79788456f * b);
-  float t = rnd<DT>(tanh_f32(c));
-  return rnd<DT>(0.5f * x) * rnd<DT>(1.0f + t);
+// Two elements at a time, so that every rounding to a 16-bit dtype is one packed conversion for
+// the pair (these kernels are bound by their instruction count: nine roundings per element).
+template <int DT> SK_DEV f32x2 gelu_new_pair(float x0, float x1) {
+  f32x2 q = rnd2<DT>(x0 * x0, x1 * x1);
+  const f32x2 x3 = rnd2<DT>(q.x * x0, q.y * x1);
+  const f32x2 a = rnd2<DT>(0.044715f * x3.x, 0.044715f * x3.y);
+  const f32x2 b = rnd2<DT>(x0 + a.x, x1 + a.y);
+  const f32x2 c = rnd2<DT>(0.79788456f * b.x, 0.79788456f * b.y);
+  const f32x2 t = rnd2<DT>(tanh_f32(c.x), tanh_f32(c.y));
+  const f32x2 h = rnd2<DT>(0.5f * x0, 0.5f * x1);
+  const f32x2 o = rnd2<DT>(1.0f + t.x, 1.0f + t.y);
+  f32x2 r = {h.x * o.x, h.y * o.y};
+  return r;
 }
-template <int DT> SK_DEV float gelu_fast_elem(float x) {
-  float a = rnd<DT>(x * 0.79788456f);
-  float b = rnd<DT>(0.044715f * x);
-  float c = rnd<DT>(b * x);
-  float e = rnd<DT>(1.0f + c);
-  float u = rnd<DT>(a * e);
-  float t = rnd<DT>(tanh_f32(u));
-  return rnd<DT>(0.5f * x) * rnd<DT>(1.0f + t);
+template <int DT> SK_DEV f32x2 gelu_fast_pair(float x0, float x1) {
+  const f32x2 a = rnd2<DT>(x0 * 0.79788456f, x1 * 0.79788456f);
+  const f32x2 b = rnd2<DT>(0.044715f * x0, 0.044715f * x1);
+  const f32x2 c = rnd2<DT>(b.x * x0, b.y * x1);
+  const f32x2 e = rnd2<DT>(1.0f + c.x, 1.0f + c.y);
+  const f32x2 u = rnd2<DT>(a.x * e.x, a.y * e.y);
+  const f32x2 t = rnd2<DT>(tanh_f32(u.x), tanh_f32(u.y));
+  const f32x2 h = rnd2<DT>(0.5f * x0, 0.5f * x1);
+  const f32x2 o = rnd2<DT>(1.0f + t.x, 1.0f + t.y);
+  f32x2 r = {h.x * o.x, h.y * o.y};
+  return r;
 }
+template <int DT> SK_DEV float gelu_new_elem(float x) { return gelu_new_pair<DT>(x, x).x; }
+template <int DT> SK_DEV float gelu_fast_elem(float x) { return gelu_fast_pair<DT>(x, x).x; }
 
 // Flat element-wise kernel: the tensor is cut into spans of kGeluSpan bytes (one
 // buffer resource each, grid.y), a workgroup handles 1 KiB of a span.  Elements
@@ -140,8 +151,11 @@ __global__ __launch_bounds__(kRowSeg) void gelu_kernel(void* __restrict__ out,
   Vec<DT> x;
   x.unpack(buf_load16<kStreamLoad>(ri, off));
 #pragma unroll
-  for (int i = 0; i < N; ++i)
-    x.f[i] = FAST ? gelu_fast_elem<DT>(x.f[i]) : gelu_new_elem<DT>(x.f[i]);
+  for (int i = 0; i < N; i += 2) {
+    const f32x2 r = FAST ? gelu_fast_pair<DT>(x.f[i], x.f[i + 1]) : gelu_new_pair<DT>(x.f[i], x.f[i + 1]);
+    x.f[i] = r.x;
+    x.f[i + 1] = r.y;
+  }
   buf_store16<kStreamStore>(ro, off, x.pack());
   if (blockIdx.x == 0 && blockIdx.y == 0) {
     const int64_t i = vec_bytes / ElemBytes<DT>::value + threadIdx.x;

@@ -190,6 +190,27 @@ def test_gelu_matches_oracle(ops, dev, dtype, name, T, d):
     assert_close_dtype(got, want, **tol)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["gelu_new", "gelu_fast"])
+def test_gelu_saturation_and_non_finite_inputs(ops, dev, dtype, name):
+    """The tanh inside is 1 - 2 / (1 + e^{2u}) with no clamp: it must saturate to +-1 through an
+    infinite or zero exponential, and NaN / infinities must come out as the arithmetic of the
+    reference's expression gives them (0.5 * -inf * (1 + -1) is NaN, for one)."""
+    vals = [0.0, -0.0, 0.5, -0.5, 3.0, -3.0, 9.0, -9.0, 20.0, -20.0, 100.0, -100.0, 1e4, -1e4,
+            float("inf"), float("-inf"), float("nan")]
+    x = torch.tensor(vals * 8, dtype=torch.float32).to(dtype).reshape(1, -1)   # 136 = 17 vectors
+    want = torch.empty_like(x)
+    getattr(c_oracle, name)(want, x)
+    got = torch.empty_like(x, device=dev)
+    getattr(ops.activation_ops, name)(got, x.to(dev))
+    got = got.cpu()
+    assert torch.equal(torch.isnan(got), torch.isnan(want))
+    sat = ~torch.isnan(want) & ((x.float().abs() >= 20.0) | (x.float() == 0.0))
+    assert torch.equal(got[sat], want[sat])   # saturated values, infinities and signed zeros: exact
+    mid = ~torch.isnan(want) & ~sat
+    assert_close_dtype(got[mid].reshape(1, -1), want[mid].reshape(1, -1), **_tol(dtype))
+
+
 # ------------------------------------------------------------------ rotary
 
 def _rope_case(ops, dev, dtype, T, nq, nkv, D, R, is_neox, packed, seed=1, prefill=None):
