@@ -166,8 +166,8 @@ int64_t sarathi_moe_align_workspace_bytes(int64_t numel, int num_experts);
  * sarathi_moe_align_block_size for callers that cannot allocate device memory or bring a
  * workspace (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
  * It has no counterpart in the reference.  Same arguments, results and error codes as
- * sarathi_moe_align_block_size without `workspace`; the scratch of the three-launch path for
- * inputs above 16 K ids is a fixed array of SARATHI_MOE_ALIGN_STATIC_SCRATCH_BYTES that lives in
+ * sarathi_moe_align_block_size without `workspace`; the scratch of the three-launch path (inputs
+ * above 32 768 ids, or above 16 384 with more than 256 experts) is a fixed array of SARATHI_MOE_ALIGN_STATIC_SCRATCH_BYTES that lives in
  * the library's device image (every GPU the library runs on holds it until the process ends).
  * The call allocates and frees nothing.  Inputs for which
  * sarathi_moe_align_workspace_bytes(numel, num_experts) exceeds that size are refused with

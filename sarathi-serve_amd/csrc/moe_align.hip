@@ -745,7 +745,7 @@ extern "C" int sarathi_moe_align_block_size_static(const void* topk_ids, int id_
                                                    int32_t* num_tokens_post_pad, int fill_pad,
                                                    void* stream) {
   using namespace sarathi_hip;
-  // 0 for inputs that take the single-workgroup path, which uses no global scratch
+  // 0 for inputs that take one of the one-launch paths, which use no global scratch
   const int64_t need = sarathi_moe_align_workspace_bytes(numel, num_experts);
   if (need > SARATHI_MOE_ALIGN_STATIC_SCRATCH_BYTES) return SARATHI_ERR_SCRATCH_LIMIT;
   int32_t* ws = nullptr;

@@ -9,7 +9,7 @@
 // torch's current HIP stream for it; (c) forwards raw pointers, sizes and
 // strides to the C ABI of include/sarathi_ops.h and turns a non-zero status
 // into a RuntimeError.  It never copies or synchronises, and allocates only the scratch
-// tensor that moe_align_block_size uses for inputs above 16 K ids and, once per (device, stream),
+// tensor that moe_align_block_size uses for inputs above 32 K ids and, once per (device, stream),
 // the four-byte completion counter of fused_topk_align.
 #include <c10/hip/HIPStream.h>
 #include <hip/hip_runtime_api.h>
