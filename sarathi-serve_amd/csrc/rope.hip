@@ -268,13 +268,16 @@ __global__ __launch_bounds__(64) void rope_append_tok_kernel(
 // 32 query + 8 key heads of 128, 1152 / 2304 / 4608 / 9216 tokens: whole token 6.1 / 8.45 / 17.3 /
 // 33.1 us, one segment 5.7 / 9.3 / 16.8 / 31.6 us; with 64 query heads (nine segments, i.e. two
 // chunks of five against nine waves of one) 4608 tokens take 31.5 against 27.3 us.
-constexpr int kMaxSegsPerWave = 5;
+// A wave's loads in flight, not its segment count, are what the limit is about: a NeoX segment is
+// two 16-byte loads per lane, a GPT-J segment one.
+constexpr int kMaxSegsPerWave = 5;       // NeoX
+constexpr int kMaxSegsPerWaveGptj = 10;
 struct RopeChunks {
   int chunks, spw;
 };
-static RopeChunks plan_rope_chunks(int64_t segs, int64_t tokens) {
+static RopeChunks plan_rope_chunks(int64_t segs, int64_t tokens, int max_segs) {
   const int64_t units = compute_units();
-  const bool whole_token = segs <= kMaxSegsPerWave && tokens >= 6 * units && tokens <= 12 * units;
+  const bool whole_token = segs <= max_segs && tokens >= 6 * units && tokens <= 12 * units;
   RopeChunks p;
   p.chunks = whole_token ? 1 : (int)(segs < 1 ? 1 : segs);
   p.spw = whole_token ? (int)(segs < 1 ? 1 : segs) : 1;
@@ -354,7 +357,8 @@ static int launch_rope_piece(const RopeLaunch& l, int64_t segs, int64_t num_toke
                              const void* value, int64_t vsb, int write_key, const KvDest* d,
                              hipStream_t st) {
   if (segs <= 0) return SARATHI_OK;
-  const RopeChunks plan = plan_rope_chunks(segs, num_tokens);
+  const RopeChunks plan =
+      plan_rope_chunks(segs, num_tokens, NEOX ? kMaxSegsPerWave : kMaxSegsPerWaveGptj);
   const bool flat = plan.chunks == 1;
   const int64_t full_z = flat ? 0 : num_tokens / kMaxGridY;
   const int64_t rem = flat ? num_tokens : num_tokens % kMaxGridY;
@@ -403,7 +407,15 @@ static int launch_rope_piece(const RopeLaunch& l, int64_t segs, int64_t num_toke
     break;
   switch (plan.spw) {
     SK_ROPE_LAUNCH(1) SK_ROPE_LAUNCH(2) SK_ROPE_LAUNCH(3) SK_ROPE_LAUNCH(4) SK_ROPE_LAUNCH(5)
-    default: return SARATHI_ERR_UNSUPPORTED;
+    default:
+      if constexpr (!NEOX) {
+        switch (plan.spw) {
+          SK_ROPE_LAUNCH(6) SK_ROPE_LAUNCH(7) SK_ROPE_LAUNCH(8) SK_ROPE_LAUNCH(9) SK_ROPE_LAUNCH(10)
+          default: return SARATHI_ERR_UNSUPPORTED;
+        }
+      } else {
+        return SARATHI_ERR_UNSUPPORTED;
+      }
   }
 #undef SK_ROPE_LAUNCH
 #undef SK_ROPE_GO

@@ -252,6 +252,9 @@ def test_rope_llama3_8b_hybrid_batch_bit_exact(ops, dev, dtype, is_neox, packed)
     (3, 2, 2, 80, 20),              # rot_dim/2 not a multiple of the vector width -> element path
     (1, 1, 1, 256, 256),
     (11, 160, 8, 128, 128),         # more heads than one pass of the block covers
+    (1700, 20, 4, 128, 128),        # one wave per token: 3 NeoX segments / 6 of interleaved pairs
+    (1700, 28, 8, 128, 128),        # 5 / 9 segments
+    (1600, 44, 4, 128, 128),        # 6 NeoX segments (one wave per segment) / 12
 ])
 def test_rope_shapes_bit_exact(ops, dev, T, nq, nkv, D, R, is_neox):
     for packed in (False, True):

@@ -211,6 +211,48 @@ def test_fused_rope_append_equals_separate_ops(ops, dev, dtype, is_neox, nq, nkv
         assert np.array_equal(_bits(ok[:n]), _bits(untouched[:n]))
 
 
+@pytest.mark.parametrize("nq,nkv,is_neox", [
+    (32, 8, False),   # ten segments of interleaved pairs in one wave
+    (28, 8, False),   # nine
+    (20, 4, False),   # six
+    (12, 4, True),    # two NeoX segments
+    (24, 8, True),    # four
+])
+@pytest.mark.parametrize("write_key", [False, True])
+def test_fused_rope_append_one_wave_per_token(ops, dev, nq, nkv, is_neox, write_key):
+    """Batches of 1536..3072 tokens take the kernel shape in which one wave covers a whole token.
+    Checked bit for bit against the two stand-alone ops (each checked against its oracle
+    elsewhere), with fewer appended rows than tokens."""
+    D, page_size, T, n = 128, 16, 1700, 1650
+    g = gen(nq * 100 + nkv)
+    pages = (n + page_size - 1) // page_size
+    table_pages = torch.randperm(pages + 3, generator=g)[:pages].to(torch.int32).to(dev)
+    indptr = torch.tensor([0, pages], dtype=torch.int32, device=dev)
+    b = torch.zeros(n, dtype=torch.int32, device=dev)
+    pos = torch.arange(n, dtype=torch.int32, device=dev)
+    positions = torch.randint(0, 4096, (T,), generator=g, dtype=torch.int64).to(dev)
+    table = cos_sin_cache(4096, D, 10000.0, torch.bfloat16).to(dev)
+    qkv = randn((T, (nq + 2 * nkv) * D), g, torch.bfloat16).to(dev)
+    cache = randn((pages + 3, 2, page_size, nkv, D), g, torch.bfloat16).to(dev)
+
+    ref, want_cache = qkv.clone(), cache.clone()
+    rq, rk, rv = ref.split([nq * D, nkv * D, nkv * D], dim=-1)
+    ops.pos_encoding_ops.rotary_embedding(positions, rq, rk, D, table, is_neox)
+    ops.kv_cache_ops.append_paged_kv_cache(rk[:n].reshape(n, nkv, D), rv[:n].reshape(n, nkv, D), b,
+                                           pos, want_cache, table_pages, indptr)
+    got, got_cache = qkv.clone(), cache.clone()
+    q, k, v = got.split([nq * D, nkv * D, nkv * D], dim=-1)
+    ops.kv_cache_ops.rotary_embedding_append_paged_kv(
+        positions, q, k, v, D, table, is_neox, b, pos, got_cache, table_pages, indptr,
+        num_append_tokens=n, write_key=write_key)
+    assert torch.equal(got_cache, want_cache)
+    assert torch.equal(q, rq) and torch.equal(v, rv) and torch.equal(k[n:], rk[n:])
+    if write_key:
+        assert torch.equal(k[:n], rk[:n])
+    else:
+        assert torch.equal(k[:n], qkv.split([nq * D, nkv * D, nkv * D], dim=-1)[1][:n])
+
+
 def test_hybrid_batch_full_size_round_trip(ops, dev):
     """Llama-3-8B hybrid batch (one 2048-token prompt chunk of a request that already holds 4096
     tokens, 256 decode requests), page size 16, through the host-side metadata builder: reading
