@@ -220,9 +220,14 @@ SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
   Vec<DT> c, s;
   c.unpack(cr);
   s.unpack(sr);
+  // Rotate every segment first and issue the stores afterwards, back to back: a wave that starts
+  // writing while its other segments (and its neighbours' rows) are still being read slows those
+  // reads down.  2304 tokens of 32 + 8 heads: 8.2 -> 7.6 us; tied at 1536 and 3072 tokens.
+#pragma unroll
+  for (int j = 0; j < SPW; ++j) rotate_slot<DT, NEOX>(xr[j], yr[j], c, s);
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int j = 0; j < SPW; ++j) {
-    rotate_slot<DT, NEOX>(xr[j], yr[j], c, s);
     bool in_place = true;
     if constexpr (APPEND) {
       const bool seg_in_a = (chunk * SPW + j) < (a_pad >> (6 - sh));
@@ -231,10 +236,10 @@ SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
       if (is_k && appended) {  // uniform
         const rsrc_t rkc = make_rsrc(reinterpret_cast<char*>(d->k_cache) + entry, kv_row_bytes);
         const rsrc_t rvc = make_rsrc(reinterpret_cast<char*>(d->v_cache) + entry, kv_row_bytes);
-        buf_store16<kKvStore>(rkc, koff[j], xr[j]);
-        if constexpr (NEOX) buf_store16<kKvStore>(rkc, koff[j] + embed_bytes, yr[j]);
-        buf_store16<kKvStore>(rvc, koff[j], vx[j]);
-        if constexpr (NEOX) buf_store16<kKvStore>(rvc, koff[j] + embed_bytes, vy[j]);
+        buf_store16<kKvStoreFused>(rkc, koff[j], xr[j]);
+        if constexpr (NEOX) buf_store16<kKvStoreFused>(rkc, koff[j] + embed_bytes, yr[j]);
+        buf_store16<kKvStoreFused>(rvc, koff[j], vx[j]);
+        if constexpr (NEOX) buf_store16<kKvStoreFused>(rvc, koff[j] + embed_bytes, vy[j]);
       }
     }
     if (in_place) {
