@@ -16,12 +16,15 @@ Infinity Cache ("cold").  `value` is the step's algorithmic bytes divided by the
 Sections (--section, comma separated, default all):
   headline  the timed chain (`value`), `per_op` for the four ops of the chain plus rms_norm alone
             (cold ring and, unless --no-warm, warm = same buffers every call) and `roofline`
-  ceiling   what the memory system gives trivial kernels at the same sizes: the library's own
-            1-load-1-store streaming kernel (moe_sum with top_k = 1) used as a copy, and the
-            launch floor (back-to-back launches of a one-row rms_norm)
+  ceiling   what the memory system gives a launch that only moves the same bytes: a plain copy in
+            every launch shape of the streaming kernels (1 to 48 KiB per one-wave workgroup), the
+            fastest shape taken as the ceiling, and the launch floor (back-to-back launches of a
+            one-row rms_norm)
   kv        paged KV-cache append alone and fused with the rotary embedding
   routing   topk_softmax, moe_align_block_size, fused_topk_align at the Mixtral shape
-  other     the CPU-sized fused_add_rms_norm [512, 4096] and the Llama-3-70B widths at T = 4608
+  other     the rest of the module surface at T = 2304, token counts off the multiples of 256
+            (T = 2248, 2560), the CPU-sized fused_add_rms_norm [512, 4096] and the Llama-3-70B
+            widths at T = 4608
   moe       fused_moe forward and its grouped GEMMs at the Mixtral-8x7B layer shape (MFMA-bound;
             beside the headline, not in it)
   cpu       `cpu_baseline`: the PyTorch CPU formulation of the same step on the host cores, and a
@@ -330,19 +333,29 @@ def main():
 
     # =========================================================================== ceiling
     if "ceiling" in want:
-        # the library's own streaming kernel with one 16-byte load and one 16-byte store per lane
-        # (moe_sum with top_k = 1 on rows of 4096 elements) as a copy of half an op's bytes in,
-        # half out
+        # What the memory system gives a launch that only moves the same number of bytes: a plain
+        # copy (half the op's bytes in, half out, same cache policies) in every launch shape the
+        # library's streaming kernels use, from 1 KiB per one-wave workgroup to 48 KiB; the fastest
+        # shape is the ceiling of that launch size.  (moe_sum with top_k = 1, the library's own
+        # copy-shaped kernel, is listed beside it.)
+        from sarathi_amd import stream_ops
         ceiling = {}
         for name in ("rms_norm", "rotary_embedding", "fused_add_rms_norm", "silu_and_mul"):
             rows = BYTES[name] // 2 // (H * BF16)
             nbytes = 2 * rows * H * BF16
             ring = ring_of(nbytes, lambda: (dev_randn((rows, 1, H)),
                                             torch.empty((rows, H), dtype=bf16, device=dev)))
+            shapes = {}
+            for kib in stream_ops.COPY_SHAPES_KIB:
+                avg, _ = time_op(lambda a: stream_ops.stream_copy(a[1], a[0], kib), ring)
+                shapes["%d KiB per wave" % kib] = round(avg, 3)
+            best = min(shapes, key=shapes.get)
             avg, med = time_op(lambda a: MOE.moe_sum(a[0], a[1]), ring)
             ceiling["copy of %s's bytes" % name] = dict(
-                frac_row(nbytes, avg), bytes=nbytes, us_event_pair_median=round(med, 3),
-                kernel="moe_sum_rows_kernel, top_k = 1: [%d, 1, %d] -> [%d, %d]" % (rows, H, rows, H))
+                frac_row(nbytes, shapes[best]), bytes=nbytes, best_shape=best,
+                kernel="stream_copy_kernel (one-wave workgroups, all loads before the first store)",
+                us_by_shape=shapes,
+                moe_sum_top1=dict(frac_row(nbytes, avg), us_event_pair_median=round(med, 3)))
             del ring
             torch.cuda.empty_cache()
         tiny_in, tiny_out = dev_randn((1, 64)), torch.empty((1, 64), dtype=bf16, device=dev)
@@ -449,10 +462,10 @@ def main():
     if "other" in want:
         # C1: the fused norm at the 512-token shape that is also the CPU-sized case; C5: the four
         # ops at Llama-3-70B widths, T = 4608 (4096-token chunk + 512 decodes), one GPU, unsharded.
-        def measure_shape(Tn, Hn, nq, nkv, dff, which):
+        def measure_shape(Tn, Hn, nq, nkv, dff, which, prefill=None):
             rows = {}
             wn = dev_randn((Hn,))
-            posn = hybrid_positions(Tn, Tn - Tn // 9, gen(4), prefill_start=4096,
+            posn = hybrid_positions(Tn, prefill or Tn - Tn // 9, gen(4), prefill_start=4096,
                                     max_pos=8192).to(dev) if any("rotary" in w for w in which) else None
             plan = {
                 "fused_add_rms_norm": (4 * Tn * Hn * BF16 + Hn * BF16,
@@ -500,6 +513,12 @@ def main():
             "[2304, 14336], rotary_embedding with interleaved (GPT-J) pairs":
                 measure_shape(T, H, NQ, NKV, DFF,
                               ["gelu_new", "gelu_fast", "rotary_embedding (GPT-J layout)"]),
+            "batches off the multiples of 256 tokens: 2048-token chunk + 200 decodes (T=2248)":
+                measure_shape(2248, H, NQ, NKV, DFF,
+                              ["fused_add_rms_norm", "rms_norm", "rotary_embedding"], prefill=PREFILL),
+            "2048-token chunk + 512 decodes (T=2560)":
+                measure_shape(2560, H, NQ, NKV, DFF,
+                              ["fused_add_rms_norm", "rms_norm", "rotary_embedding"], prefill=PREFILL),
             "fused_add_rms_norm [512, 4096] (CPU-sized case)":
                 measure_shape(512, 4096, 32, 8, 14336, ["fused_add_rms_norm"]),
             "Llama-3-70B widths, T=4608: norm [4608, 8192], rope q[4608, 8192] k[4608, 1024], "

@@ -341,6 +341,16 @@ int sarathi_rotary_embedding_append_paged_kv(
     int64_t page_stride, int64_t entry_stride, int is_neox, int write_key, int dtype,
     void* stream);
 
+/*
+ * Measurement aid with no counterpart in the reference: a device-to-device copy of `bytes` bytes
+ * (a multiple of 16, both pointers 16-byte aligned, below 4 GiB) launched the way this library's
+ * streaming ops are -- one-wave workgroups that walk memory linearly, `kib_per_wave` 16-byte loads
+ * per lane issued before the first of as many stores (1, 2, 4, 8, 12, 16, 18, 24, 36 or 48), the
+ * same cache policies.  bench.py times it at each op's byte count and reports the fastest shape as
+ * that launch size's ceiling.
+ */
+int sarathi_stream_copy(void* dst, const void* src, int64_t bytes, int kib_per_wave, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

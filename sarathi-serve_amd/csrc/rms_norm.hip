@@ -104,8 +104,13 @@ __global__ __launch_bounds__(64 * WAVES) void rms_norm_row_kernel(
 template <int DT, int VPL, int R, bool FUSED>
 __global__ __launch_bounds__(64) void rms_norm_wave_rows_kernel(
     void* out, void* in_or_res, const void* __restrict__ weight, float eps, uint32_t row_bytes,
-    float hidden_f, int64_t out_stride_bytes, int64_t in_stride_bytes, int64_t num_rows) {
+    float hidden_f, uint32_t out_stride_vecs, uint32_t in_stride_vecs, uint32_t num_rows) {
+  // Twelve dwords of arguments: all of them are preloaded into scalar registers at wave launch
+  // (the hardware preloads at most 14), so the first load waits for no argument fetch.  With the
+  // strides as 64-bit byte counts the row count fell outside and every wave spent about a
+  // microsecond on a scalar load before its first row load.  Strides are in 16-byte vectors.
   constexpr int N = VecElems<DT>::value;
+  const int64_t out_stride_bytes = (int64_t)out_stride_vecs * 16, in_stride_bytes = (int64_t)in_stride_vecs * 16;
   const int64_t row0 = (int64_t)blockIdx.x * R;
   const rsrc_t rw = make_rsrc(weight, row_bytes);
   const uint32_t off0 = threadIdx.x * 16u;
@@ -224,6 +229,7 @@ __global__ __launch_bounds__(64) void fused_add_rms_norm_wave_kernel(
   for (int j = 0; j < VPL; ++j) buf_store16<kStreamStore>(rout, off0 + j * 1024u, hid[j]);
 }
 
+
 // Any shape / alignment: one 256-thread block per row, element-wise accesses,
 // the row re-read from cache for the second pass.
 template <int DT, bool FUSED>
@@ -273,16 +279,11 @@ static int launch_rms(void* out, void* in, const void* w, float eps, int64_t T, 
 #define SK_RMS_CASE(WAVES, VPL)                                                               \
   hipLaunchKernelGGL((rms_norm_row_kernel<DT, WAVES, VPL, FUSED>), grid, dim3(64 * WAVES), 0, \
                      st, out, in, w, eps, row_bytes, hidden_f, out_stride * EB, in_stride * EB)
-  // Fused op on rows of 257..512 vectors (H = 4096 at 16 bits): two or three rows per one-wave
-  // workgroup where the row count makes that come out even over the compute units.  (The plain
-  // norm gains nothing from it with write-through stores, 7.1 us either way at 2304 x 4096; with
-  // write-back non-temporal stores it gains 4 % on cold inputs and loses 35 % on inputs that are
-  // still in the memory-side cache, which is how the reference's callers present them.)
   // Fused op on rows of 129..512 vectors in mid-sized batches (4 to 12 rows per compute unit): one
-  // wave per row with the stores held back.  Measured against the shapes below at H = 4096 bf16:
-  // 1280 rows 8.3 -> 7.5 us, 2048 11.9 -> 11.3, 2248 12.7 -> 12.2, 2304 12.7 -> 12.4, 2560 15.5 ->
-  // 14.5; smaller batches want more waves per row, and from 3072 rows on several rows per wave or
-  // plain streaming win (3072: 16.8 against 17.8 us).
+  // wave per row with the stores held back, a grid with no row counts it prefers.  Against the
+  // shapes below at H = 4096 bf16, on separately allocated tensors: 2048 rows 11.9 -> 11.4 us,
+  // 2248 12.9 -> 12.7, 2304 12.9 -> 12.9, 2560 15.8 -> 14.6.  Smaller batches want more waves per
+  // row; from 3072 rows on several rows per wave win (3072: 16.8 against 17.8 us).
   if constexpr (FUSED) {
     const int64_t units = compute_units();
     if (nvec > 128 && nvec <= 512 && T > 4 * units && T < 12 * units) {
@@ -295,12 +296,18 @@ static int launch_rms(void* out, void* in, const void* w, float eps, int64_t T, 
       return launch_status();
     }
   }
-  if (FUSED && nvec > 256 && nvec <= 512) {
+  // Fused op on rows of 257..512 vectors outside that range: two or three rows per one-wave
+  // workgroup where the row count makes that come out even over the compute units.  (The plain
+  // norm gains nothing from several rows per wave, from holding its stores back, or from two
+  // waves per row: 7.1, 7.3, 7.5, 7.7 us at 2304 x 4096.)
+  if (FUSED && nvec > 256 && nvec <= 512 && out_stride / N <= 0xffffffffLL &&
+      in_stride / N <= 0xffffffffLL) {
     const int rows_per_wg = pick_rows_per_workgroup(T, 3);
     const dim3 rgrid((unsigned)((T + rows_per_wg - 1) / rows_per_wg));
 #define SK_RMS_ROWS(R)                                                                           \
   hipLaunchKernelGGL((rms_norm_wave_rows_kernel<DT, 8, R, FUSED>), rgrid, dim3(64), 0, st, out,  \
-                     in, w, eps, row_bytes, hidden_f, out_stride * EB, in_stride * EB, T)
+                     in, w, eps, row_bytes, hidden_f, (uint32_t)(out_stride / N),                 \
+                     (uint32_t)(in_stride / N), (uint32_t)T)
     if (rows_per_wg == 3) {
       SK_RMS_ROWS(3);
       return launch_status();

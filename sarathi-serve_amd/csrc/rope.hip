@@ -166,13 +166,14 @@ SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
   const uint32_t slot = threadIdx.x & ((1u << sh) - 1u);
   const uint32_t h0 = chunk * (uint32_t)(SPW << (6 - sh)) + (threadIdx.x >> sh);
 
-  bool appended = false;
-  if constexpr (APPEND) appended = tok < d->nnz;  // uniform over the wave
   const uint32_t kv_row_bytes = (a_is_key ? heads_a : heads_b) * head_bytes;
 
   u32x4 xr[SPW], yr[SPW], vx[SPW], vy[SPW];
   uint32_t xoff[SPW];   // offset of the lane's x vector from A's row
   uint32_t koff[SPW];   // APPEND: the same offset inside the k / v row
+  // The query / key loads need nothing beyond the kernel arguments that the hardware preloads into
+  // scalar registers (the first 14 dwords), so they leave before the wave has waited for anything;
+  // the value loads and the append bookkeeping read later arguments and follow them.
 #pragma unroll
   for (int j = 0; j < SPW; ++j) {
     const uint32_t h = h0 + (uint32_t)(j << (6 - sh));
@@ -180,13 +181,19 @@ SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
     const bool in_a = h < heads_a, in_b = hb < heads_b;
     const uint32_t row_off = (in_a ? h : hb) * head_bytes + slot * 16u;
     xoff[j] = (in_a || in_b) ? row_off + (in_a ? 0u : delta) : kClipped;
+    koff[j] = (in_a || in_b) ? row_off : kClipped;
     xr[j] = buf_load16<kStreamLoad>(r, xoff[j]);
     if constexpr (NEOX) yr[j] = buf_load16<kStreamLoad>(r, xoff[j] + embed_bytes);
-    if constexpr (APPEND) {
+  }
+  bool appended = false;
+  if constexpr (APPEND) {
+    __builtin_amdgcn_sched_barrier(0);
+    appended = tok < d->nnz;  // uniform over the wave
+#pragma unroll
+    for (int j = 0; j < SPW; ++j) {
       // a segment lies wholly in A's padded span or wholly in B's: uniform
       const bool seg_in_a = (chunk * SPW + j) < (a_pad >> (6 - sh));
       const bool is_k = seg_in_a == a_is_key;
-      koff[j] = (in_a || in_b) ? row_off : kClipped;
       if (is_k && appended) {
         const rsrc_t rv = make_rsrc(
             reinterpret_cast<const char*>(value) + tok * v_stride_bytes, kv_row_bytes);
@@ -222,7 +229,8 @@ SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
   s.unpack(sr);
   // Rotate every segment first and issue the stores afterwards, back to back: a wave that starts
   // writing while its other segments (and its neighbours' rows) are still being read slows those
-  // reads down.  2304 tokens of 32 + 8 heads: 8.2 -> 7.6 us; tied at 1536 and 3072 tokens.
+  // reads down.  2048-2560 tokens of 32 + 8 heads: 7-9 % faster (2304: 8.2 -> 7.6 us); within 4 %
+  // either way at 1536 and 3072 tokens.
 #pragma unroll
   for (int j = 0; j < SPW; ++j) rotate_slot<DT, NEOX>(xr[j], yr[j], c, s);
   __builtin_amdgcn_sched_barrier(0);

@@ -667,11 +667,26 @@ void moe_grouped_gemm(torch::Tensor& a, torch::Tensor& b, torch::Tensor& c,
            op);
 }
 
+// plain copy in the launch shapes of the streaming ops (bench.py's ceiling)
+void stream_copy(torch::Tensor& dst, torch::Tensor& src, int64_t kib_per_wave) {
+  const char* op = "stream_copy";
+  check_gpu(src, src, op, "src");
+  check_gpu(dst, src, op, "dst");
+  TORCH_CHECK(dst.is_contiguous() && src.is_contiguous(), op, ": tensors must be contiguous");
+  TORCH_CHECK(dst.nbytes() == src.nbytes(), op, ": dst and src must hold the same number of bytes");
+  LaunchScope scope(src);
+  raise_on(sarathi_stream_copy(dst.data_ptr(), src.data_ptr(), (int64_t)src.nbytes(),
+                               (int)kib_per_wave, scope.stream),
+           op);
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "gfx950 HIP implementation of Sarathi-Serve's csrc op library";
   m.def("abi_version", &sarathi_ops_abi_version);
+  m.def("stream_copy", &stream_copy,
+        "device-to-device copy in the launch shapes of the streaming ops (measurement aid)");
   // layernorm_ops
   m.def("rms_norm", &rms_norm, "out = rms_norm(input) * weight");
   m.def("fused_add_rms_norm", &fused_add_rms_norm,

@@ -194,3 +194,26 @@ def test_ops_under_the_reference_package_name(tmp_path, dev):
         sys.path.remove(str(tmp_path))
         for m in [m for m in sys.modules if m == "sarathi" or m.startswith("sarathi.")]:
             del sys.modules[m]
+
+
+@pytest.mark.parametrize("nbytes", [16, 1024 + 48, 24 * 1024, 3 * 36 * 1024 + 16, 18874368])
+def test_stream_copy_every_launch_shape_byte_exact(lib, dev, nbytes):
+    """The copy that bench.py uses as the ceiling: every launch shape moves exactly `nbytes` bytes
+    (sizes that end inside a wave's span, inside a vector row, and the 2304 x 4096 bf16 tensor) and
+    touches nothing beyond them."""
+    from sarathi_amd import stream_ops
+    lib.sarathi_stream_copy.argtypes = [abi.vp, abi.vp, abi.i64, abi.ci, abi.vp]
+    lib.sarathi_stream_copy.restype = abi.ci
+    g = torch.Generator().manual_seed(nbytes)
+    src = torch.randint(0, 256, (nbytes,), generator=g, dtype=torch.uint8).to(dev)
+    for kib in stream_ops.COPY_SHAPES_KIB:
+        buf = torch.full((nbytes + 4096,), 0xA5, dtype=torch.uint8, device=dev)
+        abi.check(lib, lib.sarathi_stream_copy(abi.ptr(buf), abi.ptr(src), nbytes, kib, abi.stream()))
+        torch.cuda.synchronize()
+        assert torch.equal(buf[:nbytes], src), "copy differs at %d KiB per wave" % kib
+        assert bool((buf[nbytes:] == 0xA5).all()), "bytes beyond the end were written"
+    out = torch.empty_like(src)
+    stream_ops.stream_copy(out, src, 24)       # through the torch front end
+    assert torch.equal(out, src)
+    assert lib.sarathi_stream_copy(abi.ptr(out), abi.ptr(src), nbytes, 5, abi.stream()) == -2
+    assert lib.sarathi_stream_copy(abi.ptr(out), abi.ptr(src), 24, 8, abi.stream()) == -1

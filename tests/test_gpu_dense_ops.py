@@ -57,15 +57,21 @@ def test_fused_add_rms_norm_matches_oracle(ops, dev, dtype, T, H):
     assert_close_dtype(gx, wx, **_tol(dtype))
 
 
-@pytest.mark.parametrize("T,H", [(2304, 4096), (2305, 4096), (1030, 4096), (2304, 3072),
-                                 (1537, 2560)])
-def test_fused_add_rms_norm_rows_per_workgroup(ops, dev, T, H):
-    """Row counts at which the launch puts two or three rows into one workgroup (2304 -> 3,
-    2305 and 1030 -> 2 with a ragged last workgroup), and widths short of the workgroup's 512
-    vectors: same results as the oracle over every row."""
+@pytest.mark.parametrize("T,H,dtype", [
+    (2304, 4096, torch.bfloat16), (2305, 4096, torch.bfloat16), (1030, 4096, torch.bfloat16),
+    (2304, 3072, torch.bfloat16), (1537, 2560, torch.bfloat16), (2248, 2048, torch.bfloat16),
+    (1500, 4096, torch.float16), (1500, 2048, torch.float32), (1100, 1032, torch.float32),
+    (3072, 4096, torch.bfloat16), (3073, 4096, torch.bfloat16), (4096, 4096, torch.bfloat16),
+    (4099, 3072, torch.float16)])
+def test_fused_add_rms_norm_rows_per_workgroup(ops, dev, T, H, dtype):
+    """The launch shapes of the fused op on rows of up to 512 vectors: one wave per row with the
+    stores held back (more than 1024 and fewer than 3072 rows: whole and ragged widths, both vector
+    counts per lane, all dtypes), and two or three rows per one-wave workgroup beyond that (3072 ->
+    3, 4096 -> 2, with ragged last workgroups).  Same results as the oracle over every row, through
+    views whose row stride differs from the width."""
     g = gen(T + H)
-    x, r = randn((T, H), g), randn((T, H), g)
-    w = randn((H,), g, mean=1.0, std=0.1)
+    x, r = randn((T, H), g, dtype), randn((T, H), g, dtype)
+    w = randn((H,), g, dtype, mean=1.0, std=0.1)
     wx, wr = x.clone(), r.clone()
     c_oracle.fused_add_rms_norm(wx, wr, w, 1e-5)
     # views into wider buffers: the row stride differs from the width
@@ -76,7 +82,7 @@ def test_fused_add_rms_norm_rows_per_workgroup(ops, dev, T, H):
     gr.copy_(r)
     ops.layernorm_ops.fused_add_rms_norm(gx, gr, w.to(dev), 1e-5)
     assert torch.equal(gr.cpu(), wr), "residual = T(x + r) must be bit-exact"
-    assert_close_dtype(gx, wx)
+    assert_close_dtype(gx, wx, **_tol(dtype))
     assert bool((gx_buf[:, H:] == 0).all()) and bool((gr_buf[:, H:] == 0).all())
 
 
