@@ -177,7 +177,9 @@ int64_t sarathi_moe_align_workspace_bytes(int64_t numel, int num_experts);
  * their launches) race on it; calls on one stream are safe.  The array's contents between calls
  * are irrelevant: every word a call reads it has written before.  This is the one entry point of
  * the library that keeps state (the per-device address of the array, looked up on the first call on
- * each device).
+ * each device).  That lookup is host work: call the entry point once, eagerly, on every device
+ * before capturing a call into a HIP graph (inputs of at most 32 768 ids never touch the array and
+ * do not trigger the lookup, so use a larger one or rely on an earlier uncaptured call).
  */
 #define SARATHI_MOE_ALIGN_STATIC_SCRATCH_BYTES (1 << 20)
 int sarathi_moe_align_block_size_static(const void* topk_ids, int id_dtype, int64_t numel,

@@ -28,6 +28,18 @@
 //
 // Each LDS counter has a single writer wave, there is no global scratch and no
 // inter-workgroup traffic, so the result is deterministic and bit-exact.
+//
+// That single workgroup (moe_align_kernel) takes inputs of up to 256 ids, more than 256 experts,
+// and id arrays that are not 16-byte aligned.  The other paths of this file, all with the same
+// results:
+//   moe_align_few_experts_kernel   up to 32 experts, 257..32768 ids: one launch of independent
+//                                  four-wave workgroups with packed register counters
+//                                  (8192 ids of 8 experts: 5.2 us)
+//   moe_align_lds_hist_kernel      33..256 experts, same scheme with LDS histograms
+//                                  (12288 ids of 64 experts: 7.4 us)
+//   count -> scan -> scatter       above 32768 ids (16384 with more than 256 experts): three
+//                                  launches over the whole GPU with a caller workspace, or with the
+//                                  file-scope array of sarathi_moe_align_block_size_static
 #include <atomic>
 
 #include "moe_align_body.h"
@@ -58,9 +70,9 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(
 // scatters its own one or two tiles with one ballot per expert.  The results do not depend on
 // how many workgroups run, and nothing is exchanged through global memory, so the sort is
 // deterministic and bit-exact.  8192 ids, 8 experts on MI355X: 8.5 us as one workgroup, 6.2 us
-// in this form with 64-bit counters and shuffle scans, and the figure in the host code below
-// with 32-bit counters, DPP folds and the expert prefix in scalar registers.  expert_ids and the padding slots are written in slices, one per
-// workgroup.
+// in this form with 64-bit counters and shuffle scans, 5.2 us with 32-bit counters, DPP folds and
+// the expert prefix in scalar registers (the shipped form).  expert_ids and the padding slots are
+// written in slices, one per workgroup.
 // ---------------------------------------------------------------------------
 constexpr int kFewMaxExperts = 32;
 // Largest input of the one-launch kernels below.  Every workgroup reads all ids, so the work
@@ -70,6 +82,14 @@ constexpr int kFewMaxExperts = 32;
 // 32768 / 256 = 128 ids.)
 constexpr int64_t kOneLaunchMaxIds = 32768;
 constexpr int kFewWaves = 4;
+// The few-experts kernel counts in byte-wide fields per lane and folds them over the wave in
+// 16-bit fields: a lane sees at most kOneLaunchMaxIds / (64 * kFewWaves) ids (plus one load's worth
+// of rounding), a wave 64 times that.  Raising the id limit or lowering the wave count past these
+// bounds would wrap a counter silently.
+static_assert(kOneLaunchMaxIds / (64 * kFewWaves) + 4 <= 255,
+              "per-lane byte counters of moe_align_few_experts_kernel would overflow");
+static_assert(kOneLaunchMaxIds / kFewWaves + 4 * 64 <= 65535,
+              "16-bit wave totals of moe_align_few_experts_kernel would overflow");
 constexpr int kFewCountBatch = 8;   // 16-byte loads in flight per lane while counting
 
 // Adds `v` over the 64 lanes of a wave; the total is valid in LANE 63 only.  Four DPP folds make

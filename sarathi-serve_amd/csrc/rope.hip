@@ -10,12 +10,12 @@
 //   GPT-J: x and y interleave, so one 16-byte vector already holds whole
 //          pairs; cos and sin come from two half-width loads.
 // 64 consecutive slots of a token's q row or of its k row (8 heads of 128 at
-// bf16) form a segment.  A workgroup is ONE wave that takes up to five
-// consecutive segments of one token's list (q segments, then k segments): at
-// Llama-3-8B's 32 + 8 heads that is the whole token, so its position and its
+// bf16) form a segment.  A workgroup is ONE wave that takes up to five NeoX
+// (ten GPT-J) consecutive segments of one token's list (q segments, then k
+// segments): at Llama-3-8B's 32 + 8 heads that is the whole token, so its position and its
 // cos/sin row are fetched once, all of its loads are in flight before the first
 // result is needed, and the launch has one workgroup per token.  (Measured on
-// MI355X at 2304 tokens: one wave per segment 9.3 us, one wave per token 8.4 us;
+// MI355X at 2304 tokens: one wave per segment 9.3 us, one wave per token 8.1 us;
 // a launch of N one-wave workgroups costs about 0.2 ns per workgroup in the
 // dispatcher alone, 3.5 us for the 11520 of the per-segment layout, and
 // multi-wave workgroups lose more to uneven compute-unit load than they gain.)
@@ -276,11 +276,14 @@ __global__ __launch_bounds__(64) void rope_append_tok_kernel(
 
 // Segments a wave takes.  One wave per segment (a grid of segments x tokens) is the general
 // shape.  A whole token per wave (a flat grid of tokens, all of the token's loads in flight at
-// once, position and cache row fetched once) wins only where that grid is six to twelve waves
-// per compute unit, which is where the 2304-token Llama-3-8B batch falls.  Measured, bf16,
-// 32 query + 8 key heads of 128, 1152 / 2304 / 4608 / 9216 tokens: whole token 6.1 / 8.45 / 17.3 /
-// 33.1 us, one segment 5.7 / 9.3 / 16.8 / 31.6 us; with 64 query heads (nine segments, i.e. two
-// chunks of five against nine waves of one) 4608 tokens take 31.5 against 27.3 us.
+// once, position and cache row fetched once, every store behind the last rotation) wins where that
+// grid is five to about ten waves per compute unit, which is where a 2048-token chunk plus its
+// decode tokens falls.  Measured on separately allocated tensors, bf16, 32 query + 8 key heads of
+// 128, cold, whole token / one segment per wave: 1024 tokens 5.2 / 5.0 us, 1280 5.8 / 5.8, 1536
+// 6.4 / 6.8, 2048 7.2 / 8.4, 2304 8.1 / 9.3, 2560 9.9 / 10.2, 2816 11.3 / 10.9, 3072 12.2 / 11.6,
+// 4096 16.0 / 14.9 (on inputs still in the memory-side cache the whole token wins throughout).
+// With 64 query heads (nine segments, i.e. two chunks of five against nine waves of one) 4608
+// tokens take 31.5 against 27.3 us.
 // A wave's loads in flight, not its segment count, are what the limit is about: a NeoX segment is
 // two 16-byte loads per lane, a GPT-J segment one.
 constexpr int kMaxSegsPerWave = 5;       // NeoX
@@ -290,7 +293,7 @@ struct RopeChunks {
 };
 static RopeChunks plan_rope_chunks(int64_t segs, int64_t tokens, int max_segs) {
   const int64_t units = compute_units();
-  const bool whole_token = segs <= max_segs && tokens >= 6 * units && tokens <= 12 * units;
+  const bool whole_token = segs <= max_segs && tokens >= 5 * units && 2 * tokens <= 21 * units;
   RopeChunks p;
   p.chunks = whole_token ? 1 : (int)(segs < 1 ? 1 : segs);
   p.spw = whole_token ? (int)(segs < 1 ? 1 : segs) : 1;

@@ -10,6 +10,7 @@ from .fused_moe_layer import FusedMoE
 from .kv_append import AppendMetadata, SequenceSlice, build_append_metadata
 from .moe_routing import fused_topk, fused_topk_and_align, grouped_topk, moe_align_block_size
 from .norm import RMSNorm
+from .op_timer import op_timer, set_op_timer_factory
 from .rotary import (DynamicNTKScalingRotaryEmbedding, LinearScalingRotaryEmbedding,
                      RotaryEmbedding, YaRNScalingRotaryEmbedding, get_rope)
 
@@ -18,4 +19,5 @@ __all__ = ["RMSNorm", "SiluAndMul", "NewGELU", "FastGELU", "get_act_fn", "Rotary
            "YaRNScalingRotaryEmbedding", "get_rope", "fused_topk", "fused_topk_and_align", "grouped_topk", "moe_align_block_size",
            "invoke_fused_moe_kernel", "fused_experts", "fused_moe", "FusedMoE", "get_default_config",
            "get_moe_configs", "try_get_optimal_moe_config", "pack_expert_weights",
-           "PackedExpertWeights", "SequenceSlice", "AppendMetadata", "build_append_metadata"]
+           "PackedExpertWeights", "SequenceSlice", "AppendMetadata", "build_append_metadata",
+           "op_timer", "set_op_timer_factory"]

@@ -19,8 +19,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, HERE)
 
 
-def main():
-    ap = argparse.ArgumentParser()
+def build_parser():
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("--experts", type=int, default=8)
     ap.add_argument("--topk", type=int, default=2)
     ap.add_argument("--hidden", type=int, default=4096)
@@ -34,7 +34,18 @@ def main():
                     help="expert weight layout the table is for")
     ap.add_argument("--device-name", type=str, default="",
                     help="device_name field of the file name; default: the GPU architecture")
-    args = ap.parse_args()
+    return ap
+
+
+def output_file_name(experts, intermediate, device_name, layout):
+    """Name of the table this run writes: the one ``get_moe_configs`` looks up for the same
+    (E, N), device name and weight layout."""
+    suffix = "" if layout == "packed" else ",layout=row_major"
+    return "E=%d,N=%d,device_name=%s%s.json" % (experts, intermediate, device_name, suffix)
+
+
+def main():
+    args = build_parser().parse_args()
 
     import torch
     from sarathi_amd import layers
@@ -83,8 +94,7 @@ def main():
     name = args.device_name or arch
     out_dir = args.out_dir or fm.CONFIG_DIR
     os.makedirs(out_dir, exist_ok=True)
-    suffix = "" if args.layout == "packed" else ",layout=row_major"
-    path = os.path.join(out_dir, "E=%d,N=%d,device_name=%s%s.json" % (E, I, name, suffix))
+    path = os.path.join(out_dir, output_file_name(E, I, name, args.layout))
     with open(path, "w") as f:
         json.dump(table, f, indent=4)
         f.write("\n")

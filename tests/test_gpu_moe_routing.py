@@ -174,6 +174,38 @@ def test_moe_align_skewed_and_empty(ops, dev):
     _check_align(*_align_both(ops, dev, ids, 8, 4, filled=True), 4)
 
 
+@pytest.mark.parametrize("E", [8, 32])
+@pytest.mark.parametrize("dtype", [torch.int32, torch.int64, torch.int8])
+def test_moe_align_largest_one_launch_input_on_one_expert(ops, dev, E, dtype):
+    """32768 ids, the largest input of the one-launch kernels, all on ONE expert: every per-lane
+    byte counter and every 16-bit wave total of the few-experts kernel reaches its maximum."""
+    for expert in (0, E - 1):
+        ids = torch.full((32768,), expert, dtype=dtype)
+        _check_align(*_align_both(ops, dev, ids, E, 64, filled=True), 64)
+    ids = torch.full((32768,), 5, dtype=dtype)
+    ids[::977] = 2                          # a few strays so that two runs exist
+    _check_align(*_align_both(ops, dev, ids, E, 16), 16)
+
+
+@pytest.mark.parametrize("dtype", [torch.int32, torch.int16, torch.int8])
+@pytest.mark.parametrize("E", [2, 8, 32])
+def test_moe_align_id_pointer_not_16_byte_aligned(ops, dev, E, dtype):
+    """The id array may start anywhere: a view that begins one element into its buffer (4, 2 or 1
+    bytes off a 16-byte boundary) takes the kernels without 16-byte id loads and gives the same
+    result, at sizes on both sides of every launch-shape boundary."""
+    g = gen(31 + E)
+    for numel in (300, 5000, 32767):
+        buf = torch.randint(0, E, (numel + 1,), generator=g, dtype=torch.int32).to(dtype)
+        ids_cpu = buf[1:].clone()
+        ids_dev = buf.to(dev)[1:]
+        assert ids_dev.data_ptr() % 16 != 0
+        ws, we, wp = _align_bufs(numel, E, 32, "cpu")
+        c_oracle.moe_align_block_size(ids_cpu, E, 32, ws, we, wp)
+        gs, ge, gp = _align_bufs(numel, E, 32, dev, fill=False)
+        ops.moe_ops.moe_align_block_size_filled(ids_dev, E, 32, gs, ge, gp)
+        _check_align((gs.cpu(), ge.cpu(), gp.cpu()), (ws, we, wp), 32)
+
+
 def test_moe_align_invariants_large(ops, dev):
     """64K tokens x top-2 (the largest chunk the reference's caller passes, fused_moe.py:437):
     non-padding entries are a permutation of 0..numel-1, each block holds one expert's tokens in

@@ -148,3 +148,64 @@ def test_override_config_block_size_is_raised_to_one_that_exists():
         assert fm.try_get_optimal_moe_config((8, 8, 64), (8, 64, 4), 2, 4, override_config=cfg) is cfg
     big = fm.try_get_optimal_moe_config((8, 8, 64), (8, 64, 4), 2, 4, override_config={"BLOCK_SIZE_M": 512})
     assert big["BLOCK_SIZE_M"] == 256
+
+
+def test_tuner_script_names_its_table_as_the_loader_looks_it_up(monkeypatch):
+    """``tune_fused_moe.py`` is the recipe for the tables under layers/configs: its argument parser
+    builds, and the file it would write is the one ``get_moe_configs`` opens for the same (E, N),
+    device name and weight layout; every committed table carries a name the script can produce."""
+    import importlib
+    import importlib.util
+    import os
+    import re
+    fm = importlib.import_module("sarathi_amd.layers.fused_moe")   # the module, not the function
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location(
+        "tune_fused_moe", os.path.join(root, "sarathi-serve_amd", "tune_fused_moe.py"))
+    tuner = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(tuner)
+    args = tuner.build_parser().parse_args(["--experts", "16", "--intermediate", "2688",
+                                            "--layout", "row_major", "--device-name", "gfx950"])
+    assert (args.experts, args.topk, args.hidden, args.iters) == (16, 2, 4096, 10)
+    assert [int(v) for v in args.batch_sizes.split(",")][:3] == [1, 2, 4]
+    monkeypatch.setattr(torch.cuda, "get_device_name", lambda *a: "gfx950")
+    for layout, packed in (("packed", True), ("row_major", False)):
+        assert tuner.output_file_name(16, 2688, "gfx950", layout) == \
+            fm.get_config_file_name(16, 2688, None, packed)
+    pat = re.compile(r"E=(\d+),N=(\d+),device_name=([^,]+)(,layout=row_major)?\.json$")
+    tables = sorted(n for n in os.listdir(fm.CONFIG_DIR) if n.endswith(".json"))
+    assert tables, "no tuned tables committed"
+    for name in tables:
+        m = pat.match(name)
+        assert m, name
+        assert name == tuner.output_file_name(int(m.group(1)), int(m.group(2)), m.group(3),
+                                              "row_major" if m.group(4) else "packed")
+
+
+def test_norm_layer_enters_the_installed_op_timer():
+    """The reference's per-op timer labels survive the layer boundary: RMSNorm enters the context
+    manager that the installed factory returns for (norm_name, layer_id), where the reference enters
+    its CudaTimer (sarathi/model_executor/layers/layernorm.py:29-32); without a factory, or without
+    a name, it is a no-op."""
+    import contextlib
+    from sarathi_amd import layers
+    seen = []
+
+    @contextlib.contextmanager
+    def timer(name, layer_id):
+        seen.append(("enter", name, layer_id))
+        yield
+        seen.append(("exit", name, layer_id))
+
+    layers.set_op_timer_factory(timer)
+    try:
+        norm = layers.RMSNorm(64, norm_name="input_layernorm", layer_id=3)
+        unnamed = layers.RMSNorm(64)
+    finally:
+        layers.set_op_timer_factory(None)
+    for layer in (norm, unnamed):
+        with pytest.raises(Exception):          # CPU tensors are refused by the op, inside the timer
+            layer(torch.zeros((2, 64), dtype=torch.bfloat16))
+    assert seen == [("enter", "input_layernorm", 3)] or \
+        seen == [("enter", "input_layernorm", 3), ("exit", "input_layernorm", 3)]
+    assert layers.op_timer("input_layernorm", 0).__class__ is contextlib.nullcontext

@@ -184,11 +184,13 @@ def test_gpu_moe_sum_any_shape(ops, dev, T, k, H, dt, pad_k, pad_h, seed):
 @pytest.mark.gpu
 @GPU
 @given(E=st.integers(1, 300), B=st.sampled_from([1, 4, 16, 64, 128]), n=st.integers(0, 3000),
-       idt=st.sampled_from([torch.uint8, torch.int16, torch.int32, torch.int64]),
+       idt=st.sampled_from([torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64]),
        seed=st.integers(0, 10 ** 6), skew=st.booleans(), fill=st.booleans())
 def test_gpu_moe_align_any_input_bitwise(ops, dev, E, B, n, idt, seed, skew, fill):
     if idt == torch.uint8:
         E = min(E, 255)
+    if idt == torch.int8:
+        E = min(E, 127)
     g = gen(seed)
     hi = max(1, E // 5) if skew else E
     ids = torch.randint(0, hi, (n,), generator=g, dtype=torch.int64).to(idt)

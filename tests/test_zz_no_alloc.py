@@ -88,3 +88,38 @@ def test_static_scratch_entry_small_inputs_and_limit(dev):
             assert rc == SCRATCH_LIMIT
             assert b"scratch" in lib.sarathi_ops_strerror(rc)
             assert p.item() == -7 and bool((s == -3).all())  # nothing was launched
+
+
+def test_static_scratch_entry_replays_in_a_hip_graph(dev):
+    """The caller this entry point exists for: after ONE eager call on the device (the first call
+    looks up the array's address, which is host work that must not fall into a capture), a call
+    above 32 768 ids is captured into a graph and replayed on new ids, with eager work and
+    synchronisation between the replays; every replay matches the oracle."""
+    lib = abi.load()
+    numel, E, B = 50_000, 16, 64
+    g = torch.Generator().manual_seed(43)
+    ids_dev = torch.zeros((numel,), dtype=torch.int32, device=dev)
+    s, e, p = abi.align_buffers(numel, E, B, dev, fill=-3)
+
+    def call(stream_ptr):
+        return lib.sarathi_moe_align_block_size_static(
+            abi.ptr(ids_dev), abi.ID_DT[torch.int32], numel, E, B, abi.ptr(s), s.numel(),
+            abi.ptr(e), e.numel(), abi.ptr(p), 1, stream_ptr)
+
+    abi.check(lib, call(abi.stream()))          # eager: resolves the scratch address on this device
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            abi.check(lib, call(abi.vp(side.cuda_stream)))
+    for _ in range(3):
+        ids = torch.randint(0, E, (numel,), generator=g, dtype=torch.int32)
+        ids_dev.copy_(ids)
+        s.fill_(-3)
+        e.fill_(-7)
+        p.fill_(-7)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        _same((s.cpu(), e.cpu(), p.cpu()), _oracle(ids, E, B), B)
