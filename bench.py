@@ -145,6 +145,9 @@ def main():
                     help="moe section: random = N(0,1) router logits (experts get unequal shares, "
                          "as in a real batch); balanced = every expert gets exactly tokens * top_k / "
                          "experts slots (no partly filled slot blocks): shows what the imbalance costs")
+    ap.add_argument("--moe-balance", choices=["on", "off"], default="on",
+                    help="moe section: spread every expert's slots evenly over its slot blocks before "
+                         "the GEMMs (the library's default) or leave moe_align_block_size's greedy fill")
     ap.add_argument("--moe-block-m", type=int, default=0,
                     help="moe section: slot-block size of the grouped GEMMs (0 = the library's choice)")
     args = ap.parse_args()
@@ -534,7 +537,9 @@ def main():
         # grouped expert GEMMs with the activation in the first one's epilogue, top-k sum) at the
         # Mixtral-8x7B layer shape, and the GEMMs on their own at 4096 tokens for both weight
         # layouts.  MFMA-bound at large batches, weight-streaming-bound at decode sizes.
+        import importlib
         from sarathi_amd import layers
+        importlib.import_module("sarathi_amd.layers.fused_moe").BALANCE_BLOCKS = args.moe_balance == "on"
         E, k, Hm, I = 8, 2, 4096, 14336
 
         def timeit_ms(fn, n=20):
@@ -596,6 +601,8 @@ def main():
                 config["BLOCK_SIZE_M"] = args.moe_block_m
             bm = config["BLOCK_SIZE_M"]
             s_ids, e_ids, p_pad = layers.moe_align_block_size(ti_m, bm, E)
+            if args.moe_balance == "on":
+                s_ids = layers.balance_blocks(s_ids, e_ids, p_pad, bm, E, Tn * k)
             if label == "packed":      # re-tile once, then drop the row-major copies
                 p1, p2 = layers.pack_expert_weights(w1), layers.pack_expert_weights(w2)
                 b1, b2, pk, wa, wb = p1.data, p2.data, True, p1, p2
@@ -621,8 +628,10 @@ def main():
         torch.cuda.empty_cache()
         out["moe_layer"] = {
             "shape": "Mixtral-8x7B MoE layer: 8 experts, top-2, hidden 4096, intermediate 14336, "
-                     "bf16, %s data, %s routing, back-to-back launches (weights warm in L2/MALL "
-                     "as far as they fit)" % (args.moe_data, args.moe_routing),
+                     "bf16, %s data, %s routing, slot blocks %s, back-to-back launches (weights "
+                     "warm in L2/MALL as far as they fit)"
+                     % (args.moe_data, args.moe_routing,
+                        "filled evenly per expert" if args.moe_balance == "on" else "filled greedily"),
             "peak": "2500 TFLOP/s dense bf16 MFMA; 8 TB/s HBM",
             "fused_moe_forward_row_major": forward, "at_4096_tokens": gemms}
 

@@ -344,6 +344,22 @@ int sarathi_rotary_embedding_append_paged_kv(
     void* stream);
 
 /*
+ * No counterpart in the reference: spreads every expert's slots evenly over the blocks that
+ * sarathi_moe_align_block_size gave it (fused_moe.py:151-204 fills them greedily, so an expert's
+ * last block is often nearly empty; such blocks cost the grouped GEMM far more than their share
+ * of the work, see csrc/moe_balance.hip).  sorted_in / expert_ids / num_tokens_post_pad are
+ * moe_align_block_size's outputs for `block_size`, padding entries equal to `pad_value` (the
+ * caller's numel).  sorted_out (another buffer of sorted_len entries) receives the same slots in
+ * the same order with an expert's ceil(cnt / granule) tiles of `granule` slots dealt to its nb
+ * blocks as evenly as they go (the first tiles % nb blocks take one tile more), padding elsewhere
+ * and from num_tokens_post_pad on; expert_ids and num_tokens_post_pad stay valid for it.
+ */
+int sarathi_moe_balance_blocks(const int32_t* sorted_in, int32_t* sorted_out,
+                               const int32_t* expert_ids, const int32_t* num_tokens_post_pad,
+                               int64_t sorted_len, int num_experts, int block_size, int pad_value,
+                               int granule, void* stream);
+
+/*
  * Measurement aid with no counterpart in the reference: a device-to-device copy of `bytes` bytes
  * (a multiple of 16, both pointers 16-byte aligned, below 4 GiB) launched the way this library's
  * streaming ops are -- one-wave workgroups that walk memory linearly, `kib_per_wave` 16-byte loads

@@ -94,6 +94,37 @@ def moe_align_block_size(topk_ids, num_experts, block_size, sorted_token_ids, ex
     num_tokens_post_pad[0] = int(cumsum[-1])
 
 
+def moe_balance_blocks(topk_ids, num_experts, block_size, granule):
+    """Expected output of the library's moe_balance_blocks (no counterpart in the reference), built
+    from the ids directly rather than from moe_align_block_size's output: expert e with cnt slots
+    gets nb = ceil(cnt / block) blocks; its ceil(cnt / granule) tiles of ``granule`` slots are dealt
+    to them as evenly as they go (the first blocks take the odd tiles), slots in ascending order,
+    padding (numel) elsewhere.  Returns (sorted_token_ids, expert_ids, num_tokens_post_pad) as
+    Python lists / int, lengths as the reference's caller sizes them
+    (sarathi/model_executor/layers/fused_moe/fused_moe.py:191-200)."""
+    flat = [int(v) for v in topk_ids.reshape(-1).tolist()]
+    numel = len(flat)
+    sorted_len = numel + num_experts * (block_size - 1)
+    sorted_ids, expert_ids = [], []
+    for e in range(num_experts):
+        mine = [i for i, v in enumerate(flat) if v == e]
+        if not mine:
+            continue
+        nb = -(-len(mine) // block_size)
+        tiles = -(-len(mine) // granule)
+        at = 0
+        for j in range(nb):
+            take = (tiles // nb + (1 if j < tiles % nb else 0)) * granule
+            part = mine[at:at + take]
+            at += take
+            sorted_ids += part + [numel] * (block_size - len(part))
+            expert_ids.append(e)
+        assert at >= len(mine)
+    post_pad = len(sorted_ids)
+    sorted_ids += [numel] * (sorted_len - post_pad)
+    return sorted_ids, expert_ids, post_pad
+
+
 def moe_grouped_gemm(A, B, C, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
                      num_valid_tokens, block_m, top_k, mul_routed_weight):
     """What the reference's Triton fused_moe_kernel computes

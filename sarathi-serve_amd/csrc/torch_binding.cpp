@@ -667,6 +667,35 @@ void moe_grouped_gemm(torch::Tensor& a, torch::Tensor& b, torch::Tensor& c,
            op);
 }
 
+// even fill of every expert's slot blocks (input: moe_align_block_size's outputs)
+void moe_balance_blocks(torch::Tensor& sorted_in, torch::Tensor& sorted_out, torch::Tensor& expert_ids,
+                        torch::Tensor& num_tokens_post_pad, int64_t num_experts, int64_t block_size,
+                        int64_t pad_value, int64_t granule) {
+  const char* op = "moe_balance_blocks";
+  check_gpu(sorted_in, sorted_in, op, "sorted_in");
+  check_gpu(sorted_out, sorted_in, op, "sorted_out");
+  check_gpu(expert_ids, sorted_in, op, "expert_ids");
+  check_gpu(num_tokens_post_pad, sorted_in, op, "num_tokens_post_pad");
+  TORCH_CHECK(sorted_in.scalar_type() == at::ScalarType::Int && sorted_out.scalar_type() == at::ScalarType::Int &&
+                  expert_ids.scalar_type() == at::ScalarType::Int &&
+                  num_tokens_post_pad.scalar_type() == at::ScalarType::Int,
+              op, ": all tensors must be int32");
+  TORCH_CHECK(sorted_in.is_contiguous() && sorted_out.is_contiguous() && expert_ids.is_contiguous() &&
+                  sorted_in.numel() == sorted_out.numel() && num_tokens_post_pad.numel() >= 1,
+              op, ": sorted_in / sorted_out must be contiguous and equally long");
+  TORCH_CHECK(sorted_in.data_ptr() != sorted_out.data_ptr(), op, ": cannot run in place");
+  TORCH_CHECK(block_size > 0 && granule > 0 && num_experts > 0, op, ": bad block_size / granule / num_experts");
+  TORCH_CHECK(expert_ids.numel() * block_size >= sorted_in.numel() - (block_size - 1), op,
+              ": expert_ids is too short for sorted_in");
+  LaunchScope scope(sorted_in);
+  raise_on(sarathi_moe_balance_blocks(sorted_in.data_ptr<int32_t>(), sorted_out.data_ptr<int32_t>(),
+                                      expert_ids.data_ptr<int32_t>(),
+                                      num_tokens_post_pad.data_ptr<int32_t>(), sorted_in.numel(),
+                                      (int)num_experts, (int)block_size, (int)pad_value, (int)granule,
+                                      scope.stream),
+           op);
+}
+
 // plain copy in the launch shapes of the streaming ops (bench.py's ceiling)
 void stream_copy(torch::Tensor& dst, torch::Tensor& src, int64_t kib_per_wave) {
   const char* op = "stream_copy";
@@ -731,6 +760,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "softmax, keep the best topk_group of num_expert_group expert groups, top-k of the rest");
   m.def("fused_topk_align", &fused_topk_align,
         "topk_softmax (+ optional renormalisation) and moe_align_block_size in one launch");
+  m.def("moe_balance_blocks", &moe_balance_blocks,
+        "spread every expert's slots evenly over its blocks (for the grouped GEMM)");
   m.def("moe_grouped_gemm", &moe_grouped_gemm,
         "C[slot] = A[slot / top_k] @ B[expert(slot)]^T over moe_align_block_size's layout",
         pybind11::arg("a"), pybind11::arg("b"), pybind11::arg("c"), pybind11::arg("topk_weights"),

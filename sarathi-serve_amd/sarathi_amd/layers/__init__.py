@@ -8,7 +8,8 @@ from .fused_moe import (PackedExpertWeights, fused_experts, fused_moe, get_defau
                         try_get_optimal_moe_config)
 from .fused_moe_layer import FusedMoE
 from .kv_append import AppendMetadata, SequenceSlice, build_append_metadata
-from .moe_routing import fused_topk, fused_topk_and_align, grouped_topk, moe_align_block_size
+from .moe_routing import (balance_blocks, fused_topk, fused_topk_and_align, grouped_topk,
+                          moe_align_block_size)
 from .norm import RMSNorm
 from .op_timer import op_timer, set_op_timer_factory
 from .rotary import (DynamicNTKScalingRotaryEmbedding, LinearScalingRotaryEmbedding,
@@ -20,4 +21,4 @@ __all__ = ["RMSNorm", "SiluAndMul", "NewGELU", "FastGELU", "get_act_fn", "Rotary
            "invoke_fused_moe_kernel", "fused_experts", "fused_moe", "FusedMoE", "get_default_config",
            "get_moe_configs", "try_get_optimal_moe_config", "pack_expert_weights",
            "PackedExpertWeights", "SequenceSlice", "AppendMetadata", "build_append_metadata",
-           "op_timer", "set_op_timer_factory"]
+           "op_timer", "set_op_timer_factory", "balance_blocks"]

@@ -17,7 +17,8 @@ from typing import Any, Dict, Optional, Tuple
 import torch
 
 from .. import activation_ops, moe_ops
-from .moe_routing import fused_topk, fused_topk_and_align, grouped_topk, moe_align_block_size
+from .moe_routing import (balance_blocks, fused_topk, fused_topk_and_align, grouped_topk,
+                          moe_align_block_size)
 
 _BLOCK_SIZES = (32, 64, 128, 256)
 
@@ -77,6 +78,9 @@ FUSED_ROUTING_MAX_SLOTS = 1024
 FUSED_ROUTING_MAX_EXPERTS = 16
 # silu_and_mul inside the gate/up GEMM's epilogue (same bits as the separate kernel)
 FUSE_SILU_AND_MUL = True
+# spread every expert's slots evenly over its blocks before the GEMMs (moe_routing.balance_blocks)
+# whenever some expert can have more than one block
+BALANCE_BLOCKS = True
 CHUNK_SIZE = 64 * 1024     # tokens per pass, as in the reference (fused_moe.py:437)
 
 
@@ -226,6 +230,9 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
         else:
             sorted_ids, expert_ids, post_padded = moe_align_block_size(
                 cur_ids, config["BLOCK_SIZE_M"], E)
+        if BALANCE_BLOCKS and config["BLOCK_SIZE_M"] >= 64 and n * topk > config["BLOCK_SIZE_M"]:
+            sorted_ids = balance_blocks(sorted_ids, expert_ids, post_padded,
+                                        config["BLOCK_SIZE_M"], E, n * topk)
         if fuse_act:
             invoke_fused_moe_kernel(cur_hidden, w1, c2, None, None, cur_w, cur_ids, sorted_ids,
                                     expert_ids, post_padded, False, topk, config,

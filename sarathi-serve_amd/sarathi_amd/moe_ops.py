@@ -22,9 +22,14 @@ fused_topk_align = _C.fused_topk_align
 # the group-limited routing the reference writes with tensor ops (fused_moe.py:377-408)
 grouped_topk = _C.grouped_topk
 
+# moe_balance_blocks(sorted_in, sorted_out, expert_ids, num_tokens_post_pad, num_experts, block_size,
+#                    pad_value, granule): moe_align_block_size's sort with every expert's slots spread
+# evenly over its blocks (no counterpart in the reference; what fused_experts feeds its GEMMs)
+moe_balance_blocks = _C.moe_balance_blocks
+
 # moe_sum(input[tokens, top_k, hidden], out[tokens, hidden]): the torch.sum over the top-k expert
 # outputs that ends fused_experts (fused_moe.py:539-543)
 moe_sum = _C.moe_sum
 
-__all__ = ["moe_sum", "topk_softmax", "moe_align_block_size", "topk_softmax_renorm",
+__all__ = ["moe_sum", "moe_balance_blocks", "topk_softmax", "moe_align_block_size", "topk_softmax_renorm",
            "moe_align_block_size_filled", "moe_grouped_gemm", "fused_topk_align", "grouped_topk"]

@@ -197,6 +197,35 @@ def test_fused_moe_forward(ops, dev, T, E, k, H, I, renorm):
     _close(xd, want, "fused_moe inplace")
 
 
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("block_m", [64, 128, 256])
+def test_fused_moe_same_bits_with_and_without_balanced_blocks(ops, dev, monkeypatch, packed, block_m):
+    """fused_experts spreads every expert's slots evenly over its blocks before the GEMMs; where a
+    slot sits inside a block does not enter its dot products, so the layer's output is bit for bit
+    the one computed on moe_align_block_size's own layout.  Experts with one, several and no
+    blocks, every block size that is balanced, both weight layouts."""
+    import importlib
+    fm = importlib.import_module("sarathi_amd.layers.fused_moe")   # the module, not the function
+    from sarathi_amd import layers
+    T, E, k, H, I = 1500, 8, 2, 256, 512
+    g = gen(77 + block_m)
+    x = randn((T, H), g, std=1.0).to(dev)
+    w1 = randn((E, 2 * I, H), g, std=H ** -0.5).to(dev)
+    w2 = randn((E, H, I), g, std=I ** -0.5).to(dev)
+    if packed:
+        w1, w2 = layers.pack_expert_weights(w1), layers.pack_expert_weights(w2)
+    gating = torch.randn((T, E), generator=g, dtype=torch.float32)
+    gating[:, 5] = -50.0                        # an expert nobody picks
+    gating[:, 2] += 1.5                         # and a popular one
+    gating = gating.to(dev)
+    cfg = {"BLOCK_SIZE_M": block_m, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 64, "GROUP_SIZE_M": 1}
+    assert fm.BALANCE_BLOCKS
+    got = layers.fused_moe(x, w1, w2, gating, k, True, override_config=cfg)
+    monkeypatch.setattr(fm, "BALANCE_BLOCKS", False)
+    want = layers.fused_moe(x, w1, w2, gating, k, True, override_config=cfg)
+    assert torch.equal(got, want)
+
+
 def test_fused_moe_with_one_launch_routing(ops, dev, monkeypatch):
     """fused_moe with the routing + slot sort done by the single fused launch (the default for small
     batches) and by the two separate kernels: same bits."""
