@@ -602,7 +602,7 @@ def main():
             bm = config["BLOCK_SIZE_M"]
             s_ids, e_ids, p_pad = layers.moe_align_block_size(ti_m, bm, E)
             if args.moe_balance == "on":
-                s_ids = layers.balance_blocks(s_ids, e_ids, p_pad, bm, E, Tn * k)
+                s_ids = layers.balance_blocks(s_ids, e_ids, p_pad, bm, E, Tn * k, packed=label == "packed")
             if label == "packed":      # re-tile once, then drop the row-major copies
                 p1, p2 = layers.pack_expert_weights(w1), layers.pack_expert_weights(w2)
                 b1, b2, pk, wa, wb = p1.data, p2.data, True, p1, p2

@@ -353,11 +353,23 @@ int sarathi_rotary_embedding_append_paged_kv(
  * the same order with an expert's ceil(cnt / granule) tiles of `granule` slots dealt to its nb
  * blocks as evenly as they go (the first tiles % nb blocks take one tile more), padding elsewhere
  * and from num_tokens_post_pad on; expert_ids and num_tokens_post_pad stay valid for it.
+ * rows_per_block = R > 1 deals the tiles over the expert's nb * R ranges of block_size / R slots
+ * instead (each range filled from its own start), for a GEMM kernel whose waves split a block's
+ * slots R ways: R = sarathi_moe_gemm_slot_rows(block_size, b_layout).  granule must divide
+ * block_size / R.
  */
 int sarathi_moe_balance_blocks(const int32_t* sorted_in, int32_t* sorted_out,
                                const int32_t* expert_ids, const int32_t* num_tokens_post_pad,
                                int64_t sorted_len, int num_experts, int block_size, int pad_value,
-                               int granule, void* stream);
+                               int granule, int rows_per_block, void* stream);
+
+/*
+ * No counterpart in the reference: how many equal ranges of a slot block the waves of the
+ * sarathi_moe_grouped_gemm kernel for (block_m, b_layout) split between them (1 or 2; each range
+ * is swept by its own waves, 32 slots at a time, and ranges without a valid slot in a tile are
+ * skipped per wave), or a negative SARATHI_ERR_* for an unsupported block_m / unknown layout.
+ */
+int sarathi_moe_gemm_slot_rows(int block_m, int b_layout);
 
 /*
  * Measurement aid with no counterpart in the reference: a device-to-device copy of `bytes` bytes

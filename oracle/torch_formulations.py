@@ -94,12 +94,13 @@ def moe_align_block_size(topk_ids, num_experts, block_size, sorted_token_ids, ex
     num_tokens_post_pad[0] = int(cumsum[-1])
 
 
-def moe_balance_blocks(topk_ids, num_experts, block_size, granule):
+def moe_balance_blocks(topk_ids, num_experts, block_size, granule, rows_per_block=1):
     """Expected output of the library's moe_balance_blocks (no counterpart in the reference), built
     from the ids directly rather than from moe_align_block_size's output: expert e with cnt slots
     gets nb = ceil(cnt / block) blocks; its ceil(cnt / granule) tiles of ``granule`` slots are dealt
     to them as evenly as they go (the first blocks take the odd tiles), slots in ascending order,
-    padding (numel) elsewhere.  Returns (sorted_token_ids, expert_ids, num_tokens_post_pad) as
+    padding (numel) elsewhere.  With rows_per_block = R the tiles are dealt to the expert's nb * R
+    ranges of block_size / R slots instead, each range filled from its own start.  Returns (sorted_token_ids, expert_ids, num_tokens_post_pad) as
     Python lists / int, lengths as the reference's caller sizes them
     (sarathi/model_executor/layers/fused_moe/fused_moe.py:191-200)."""
     flat = [int(v) for v in topk_ids.reshape(-1).tolist()]
@@ -112,13 +113,14 @@ def moe_balance_blocks(topk_ids, num_experts, block_size, granule):
             continue
         nb = -(-len(mine) // block_size)
         tiles = -(-len(mine) // granule)
+        ranges, width = nb * rows_per_block, block_size // rows_per_block
         at = 0
-        for j in range(nb):
-            take = (tiles // nb + (1 if j < tiles % nb else 0)) * granule
+        for j in range(ranges):
+            take = (tiles // ranges + (1 if j < tiles % ranges else 0)) * granule
             part = mine[at:at + take]
             at += take
-            sorted_ids += part + [numel] * (block_size - len(part))
-            expert_ids.append(e)
+            sorted_ids += part + [numel] * (width - len(part))
+        expert_ids += [e] * nb
         assert at >= len(mine)
     post_pad = len(sorted_ids)
     sorted_ids += [numel] * (sorted_len - post_pad)

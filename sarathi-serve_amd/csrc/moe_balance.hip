@@ -15,6 +15,13 @@
 // expert's slots, expert_ids and num_tokens_post_padded unchanged; the GEMM's results are bit for
 // bit the same (a slot's dot products do not depend on where in a block the slot sits).  No
 // counterpart in the reference; fused_experts applies it to its own, internal copy of the sort.
+//
+// A GEMM workgroup whose waves split the block's slots between them (two wave rows of 128 slots at
+// 256-slot blocks) is done when its fuller row is: a block of 224 slots laid out from its start is
+// 4 + 3 tiles and costs as much as a full one.  With rows_per_block = R the deal is over the
+// expert's nb * R row ranges of block / R slots, each filled from its own start: 1030 slots over
+// 5 blocks x 2 rows are 4 4 | 4 3 | 3 3 | 3 3 | 3 3 tiles, 17 tile times instead of 20 (16 if the
+// expert had 1024 slots).
 #include "vec16.h"
 #include "launch.h"
 
@@ -25,7 +32,7 @@ namespace sarathi_hip {
 __global__ __launch_bounds__(256) void moe_balance_blocks_kernel(
     const int32_t* __restrict__ sorted_in, int32_t* __restrict__ sorted_out,
     const int32_t* __restrict__ expert_ids, const int32_t* __restrict__ post_pad,
-    int64_t sorted_len, int num_experts, int block, int pad_value, int granule) {
+    int64_t sorted_len, int num_experts, int block, int pad_value, int granule, int rows) {
   __shared__ int first_blk, last_blk, valid_last;
   const int tid = threadIdx.x;
   int64_t end = *post_pad;
@@ -63,14 +70,15 @@ __global__ __launch_bounds__(256) void moe_balance_blocks_kernel(
   if (c) atomicAdd(&valid_last, c);
   __syncthreads();
   const int cnt = (nb - 1) * block + valid_last;
-  // the expert's slots in whole tiles of `granule`, dealt to its blocks as evenly as they go:
-  // the first `extra` blocks take one tile more than the others
+  // the expert's slots in whole tiles of `granule`, dealt to the row ranges of its blocks as evenly
+  // as they go: the first `extra` ranges take one tile more than the others
+  const int range = block / rows, ranges = nb * rows;
   const int tiles = (cnt + granule - 1) / granule;
-  const int base_tiles = tiles / nb, extra = tiles - base_tiles * nb;
+  const int base_tiles = tiles / ranges, extra = tiles - base_tiles * ranges;
   for (int i = tid; i < nb * block; i += 256) {
-    const int j = i / block, off = i - j * block;
-    const int mine = (base_tiles + (j < extra ? 1 : 0)) * granule;            // slots of block j
-    const int before = (j * base_tiles + (j < extra ? j : extra)) * granule;  // slots of blocks < j
+    const int j = i / range, off = i - j * range;
+    const int mine = (base_tiles + (j < extra ? 1 : 0)) * granule;            // slots of range j
+    const int before = (j * base_tiles + (j < extra ? j : extra)) * granule;  // slots of ranges < j
     const int r = before + off;
     sorted_out[base + i] = (off < mine && r < cnt) ? sorted_in[base + r] : pad_value;
   }
@@ -82,9 +90,10 @@ extern "C" int sarathi_moe_balance_blocks(const int32_t* sorted_in, int32_t* sor
                                           const int32_t* expert_ids,
                                           const int32_t* num_tokens_post_pad, int64_t sorted_len,
                                           int num_experts, int block_size, int pad_value,
-                                          int granule, void* stream) {
+                                          int granule, int rows_per_block, void* stream) {
   using namespace sarathi_hip;
-  if (sorted_len < 0 || num_experts <= 0 || block_size <= 0 || granule <= 0)
+  if (sorted_len < 0 || num_experts <= 0 || block_size <= 0 || granule <= 0 || rows_per_block <= 0 ||
+      block_size % rows_per_block != 0 || (block_size / rows_per_block) % granule != 0)
     return SARATHI_ERR_INVALID_ARG;
   if (sorted_len == 0) return SARATHI_OK;
   if (!sorted_in || !sorted_out || !expert_ids || !num_tokens_post_pad || sorted_in == sorted_out)
@@ -92,6 +101,6 @@ extern "C" int sarathi_moe_balance_blocks(const int32_t* sorted_in, int32_t* sor
   if (num_experts > 1024 || sorted_len > 0x7fffffffLL) return SARATHI_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(moe_balance_blocks_kernel, dim3((unsigned)num_experts + 1), dim3(256), 0,
                      (hipStream_t)stream, sorted_in, sorted_out, expert_ids, num_tokens_post_pad,
-                     sorted_len, num_experts, block_size, pad_value, granule);
+                     sorted_len, num_experts, block_size, pad_value, granule, rows_per_block);
   return launch_status();
 }

@@ -308,6 +308,17 @@ int launch_moe_gemm_wide(MoeGemmArgs g, int64_t out_cols, int block_m, int epilo
 
 }  // namespace sarathi_hip
 
+// Ranges of a slot block that separate waves sweep: the four-wave kernel for row-major weights has
+// two wave rows at every block size, the kernel of this file only in its eight-wave form.
+extern "C" int sarathi_moe_gemm_slot_rows(int block_m, int b_layout) {
+  if (b_layout != SARATHI_MOE_B_ROW_MAJOR && b_layout != SARATHI_MOE_B_PACKED)
+    return SARATHI_ERR_INVALID_ARG;
+  if (block_m != 32 && block_m != 64 && block_m != 128 && block_m != 256)
+    return SARATHI_ERR_UNSUPPORTED;
+  if (b_layout == SARATHI_MOE_B_ROW_MAJOR) return block_m >= 64 ? 2 : 1;
+  return block_m == 256 ? 2 : 1;
+}
+
 extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
                                         const float* topk_weights,
                                         const int32_t* sorted_token_ids,

@@ -670,7 +670,7 @@ void moe_grouped_gemm(torch::Tensor& a, torch::Tensor& b, torch::Tensor& c,
 // even fill of every expert's slot blocks (input: moe_align_block_size's outputs)
 void moe_balance_blocks(torch::Tensor& sorted_in, torch::Tensor& sorted_out, torch::Tensor& expert_ids,
                         torch::Tensor& num_tokens_post_pad, int64_t num_experts, int64_t block_size,
-                        int64_t pad_value, int64_t granule) {
+                        int64_t pad_value, int64_t granule, int64_t rows_per_block) {
   const char* op = "moe_balance_blocks";
   check_gpu(sorted_in, sorted_in, op, "sorted_in");
   check_gpu(sorted_out, sorted_in, op, "sorted_out");
@@ -684,7 +684,9 @@ void moe_balance_blocks(torch::Tensor& sorted_in, torch::Tensor& sorted_out, tor
                   sorted_in.numel() == sorted_out.numel() && num_tokens_post_pad.numel() >= 1,
               op, ": sorted_in / sorted_out must be contiguous and equally long");
   TORCH_CHECK(sorted_in.data_ptr() != sorted_out.data_ptr(), op, ": cannot run in place");
-  TORCH_CHECK(block_size > 0 && granule > 0 && num_experts > 0, op, ": bad block_size / granule / num_experts");
+  TORCH_CHECK(block_size > 0 && granule > 0 && num_experts > 0 && rows_per_block > 0 &&
+                  block_size % rows_per_block == 0 && (block_size / rows_per_block) % granule == 0,
+              op, ": bad block_size / granule / rows_per_block / num_experts");
   TORCH_CHECK(expert_ids.numel() * block_size >= sorted_in.numel() - (block_size - 1), op,
               ": expert_ids is too short for sorted_in");
   LaunchScope scope(sorted_in);
@@ -692,7 +694,7 @@ void moe_balance_blocks(torch::Tensor& sorted_in, torch::Tensor& sorted_out, tor
                                       expert_ids.data_ptr<int32_t>(),
                                       num_tokens_post_pad.data_ptr<int32_t>(), sorted_in.numel(),
                                       (int)num_experts, (int)block_size, (int)pad_value, (int)granule,
-                                      scope.stream),
+                                      (int)rows_per_block, scope.stream),
            op);
 }
 
@@ -761,7 +763,17 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("fused_topk_align", &fused_topk_align,
         "topk_softmax (+ optional renormalisation) and moe_align_block_size in one launch");
   m.def("moe_balance_blocks", &moe_balance_blocks,
-        "spread every expert's slots evenly over its blocks (for the grouped GEMM)");
+        "spread every expert's slots evenly over its blocks (for the grouped GEMM)",
+        pybind11::arg("sorted_in"), pybind11::arg("sorted_out"), pybind11::arg("expert_ids"),
+        pybind11::arg("num_tokens_post_pad"), pybind11::arg("num_experts"), pybind11::arg("block_size"),
+        pybind11::arg("pad_value"), pybind11::arg("granule"), pybind11::arg("rows_per_block") = 1);
+  m.def("moe_gemm_slot_rows", [](int64_t block_m, bool b_packed) {
+          const int r = sarathi_moe_gemm_slot_rows((int)block_m, b_packed ? SARATHI_MOE_B_PACKED
+                                                                          : SARATHI_MOE_B_ROW_MAJOR);
+          raise_on(r < 0 ? r : SARATHI_OK, "moe_gemm_slot_rows");
+          return (int64_t)r;
+        },
+        "ranges of a slot block that separate waves of the grouped GEMM kernel sweep (1 or 2)");
   m.def("moe_grouped_gemm", &moe_grouped_gemm,
         "C[slot] = A[slot / top_k] @ B[expert(slot)]^T over moe_align_block_size's layout",
         pybind11::arg("a"), pybind11::arg("b"), pybind11::arg("c"), pybind11::arg("topk_weights"),

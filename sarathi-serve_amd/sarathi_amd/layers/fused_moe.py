@@ -232,7 +232,8 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
                 cur_ids, config["BLOCK_SIZE_M"], E)
         if BALANCE_BLOCKS and config["BLOCK_SIZE_M"] >= 64 and n * topk > config["BLOCK_SIZE_M"]:
             sorted_ids = balance_blocks(sorted_ids, expert_ids, post_padded,
-                                        config["BLOCK_SIZE_M"], E, n * topk)
+                                        config["BLOCK_SIZE_M"], E, n * topk,
+                                        packed=isinstance(w1, PackedExpertWeights))
         if fuse_act:
             invoke_fused_moe_kernel(cur_hidden, w1, c2, None, None, cur_w, cur_ids, sorted_ids,
                                     expert_ids, post_padded, False, topk, config,

@@ -63,15 +63,19 @@ GEMM_TILE_SLOTS = 32   # slots of one matrix-core tile of the grouped GEMM kerne
 
 def balance_blocks(sorted_token_ids: torch.Tensor, expert_ids: torch.Tensor,
                    num_tokens_post_padded: torch.Tensor, block_size: int, num_experts: int,
-                   numel: int) -> torch.Tensor:
+                   numel: int, packed: bool = False) -> torch.Tensor:
     """``moe_align_block_size``'s ``sorted_token_ids`` with every expert's slots spread evenly over
     its blocks instead of filling them one after the other (no counterpart in the reference; the
     grouped GEMM runs 8-10 % faster on it when experts have a nearly empty last block, with
     bit-identical results).  ``expert_ids`` and ``num_tokens_post_padded`` stay valid for the
-    returned tensor; ``numel`` is the padding value (``topk_ids.numel()``)."""
+    returned tensor; ``numel`` is the padding value (``topk_ids.numel()``).  ``packed`` names the
+    weight layout of the GEMM that will read the result: the kernels differ in how their waves
+    split a block's slots, and the deal follows that split."""
     out = torch.empty_like(sorted_token_ids)
+    rows = moe_ops.moe_gemm_slot_rows(block_size, packed)
     moe_ops.moe_balance_blocks(sorted_token_ids, out, expert_ids, num_tokens_post_padded,
-                               num_experts, block_size, numel, min(GEMM_TILE_SLOTS, block_size))
+                               num_experts, block_size, numel,
+                               min(GEMM_TILE_SLOTS, block_size // rows), rows)
     return out
 
 

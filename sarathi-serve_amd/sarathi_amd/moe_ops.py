@@ -23,13 +23,16 @@ fused_topk_align = _C.fused_topk_align
 grouped_topk = _C.grouped_topk
 
 # moe_balance_blocks(sorted_in, sorted_out, expert_ids, num_tokens_post_pad, num_experts, block_size,
-#                    pad_value, granule): moe_align_block_size's sort with every expert's slots spread
-# evenly over its blocks (no counterpart in the reference; what fused_experts feeds its GEMMs)
+#                    pad_value, granule, rows_per_block=1): moe_align_block_size's sort with every
+# expert's slots spread evenly over its blocks, or over the rows_per_block equal ranges of each block
+# (no counterpart in the reference; what fused_experts feeds its GEMMs)
 moe_balance_blocks = _C.moe_balance_blocks
+# moe_gemm_slot_rows(block_m, b_packed): the rows_per_block that suits moe_grouped_gemm's kernel
+moe_gemm_slot_rows = _C.moe_gemm_slot_rows
 
 # moe_sum(input[tokens, top_k, hidden], out[tokens, hidden]): the torch.sum over the top-k expert
 # outputs that ends fused_experts (fused_moe.py:539-543)
 moe_sum = _C.moe_sum
 
-__all__ = ["moe_sum", "moe_balance_blocks", "topk_softmax", "moe_align_block_size", "topk_softmax_renorm",
+__all__ = ["moe_sum", "moe_balance_blocks", "moe_gemm_slot_rows", "topk_softmax", "moe_align_block_size", "topk_softmax_renorm",
            "moe_align_block_size_filled", "moe_grouped_gemm", "fused_topk_align", "grouped_topk"]

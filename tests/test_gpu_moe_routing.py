@@ -351,13 +351,15 @@ def test_grouped_topk_matches_formulation(ops, dev, T, E, k, G, keep, renorm):
     assert torch.allclose(gw.cpu(), ww, rtol=0, atol=1e-6)
 
 
+@pytest.mark.parametrize("rows", [1, 2])
 @pytest.mark.parametrize("numel,E,B", [(8192, 8, 256), (8192, 8, 64), (2000, 8, 128), (40000, 64, 256),
                                        (300, 4, 64), (5, 8, 64), (9000, 3, 256), (1024, 1, 256)])
-def test_moe_balance_blocks_spreads_every_expert_evenly(ops, dev, numel, E, B):
+def test_moe_balance_blocks_spreads_every_expert_evenly(ops, dev, numel, E, B, rows):
     """moe_balance_blocks on moe_align_block_size's output against the direct construction from
     the ids (oracle.torch_formulations.moe_balance_blocks): same blocks per expert, an expert's
-    slots in unchanged order spread over them in multiples of the GEMM's 32-slot tile, padding
-    elsewhere and beyond num_tokens_post_pad; skewed and empty experts included."""
+    slots in unchanged order spread over them (or over the two halves of each) in multiples of the
+    GEMM's 32-slot tile, padding elsewhere and beyond num_tokens_post_pad; skewed and empty experts
+    included."""
     from oracle import torch_formulations as tf
     g = gen(numel + E)
     ids = torch.randint(0, E, (numel,), generator=g, dtype=torch.int32)
@@ -366,11 +368,23 @@ def test_moe_balance_blocks_spreads_every_expert_evenly(ops, dev, numel, E, B):
     gs, ge, gp = _align_bufs(numel, E, B, dev, fill=False)
     ops.moe_ops.moe_align_block_size_filled(ids.to(dev), E, B, gs, ge, gp)
     out = torch.full_like(gs, -5)
-    ops.moe_ops.moe_balance_blocks(gs, out, ge, gp, E, B, numel, 32)
-    want_sorted, want_experts, want_pad = tf.moe_balance_blocks(ids, E, B, 32)
+    ops.moe_ops.moe_balance_blocks(gs, out, ge, gp, E, B, numel, 32, rows)
+    want_sorted, want_experts, want_pad = tf.moe_balance_blocks(ids, E, B, 32, rows)
     assert int(gp.item()) == want_pad
     assert out.cpu().tolist() == want_sorted
     assert ge.cpu()[:want_pad // B].tolist() == want_experts
-    # the layers' wrapper returns the same tensor
+    # the layers' wrapper returns the same tensor for the weight layout whose kernel splits so
     from sarathi_amd import layers
-    assert torch.equal(layers.balance_blocks(gs, ge, gp, B, E, numel), out)
+    for packed in (False, True):
+        if ops.moe_ops.moe_gemm_slot_rows(B, packed) == rows:
+            assert torch.equal(layers.balance_blocks(gs, ge, gp, B, E, numel, packed=packed), out)
+
+
+def test_moe_gemm_slot_rows_table(ops):
+    """Row-major weights: two wave rows from 64-slot blocks on; packed weights: only the eight-wave
+    kernel at 256-slot blocks; anything but 32 / 64 / 128 / 256 is refused."""
+    rows = ops.moe_ops.moe_gemm_slot_rows
+    assert [rows(b, False) for b in (32, 64, 128, 256)] == [1, 2, 2, 2]
+    assert [rows(b, True) for b in (32, 64, 128, 256)] == [1, 1, 1, 2]
+    with pytest.raises(RuntimeError):
+        rows(48, False)
