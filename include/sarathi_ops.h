@@ -86,6 +86,12 @@ int sarathi_silu_and_mul(void* out, const void* input, int64_t num_tokens, int64
  * Replace gelu_new(out, input) and gelu_fast(out, input):
  * csrc/activation.cpp:7-28, csrc/activation_kernels.cu:86-114.
  * Contiguous [num_tokens, d] in and out.
+ * 16-bit dtypes, 12 Mi elements or more: the result is read from a table of the op over all
+ * 65536 bit patterns (same bits as the arithmetic path).  The library keeps the four tables
+ * (two ops x two dtypes, 128 KiB each) in a file-scope device array; the first such call on a
+ * device launches the kernel that fills the table on its stream, and until that kernel has
+ * finished, calls on other streams and calls under stream capture use the arithmetic path.
+ * Nothing is allocated on the device and nothing waits.
  */
 int sarathi_gelu_new(void* out, const void* input, int64_t num_tokens, int64_t d, int dtype,
                      void* stream);

@@ -277,11 +277,12 @@ __global__ __launch_bounds__(64) void rope_append_tok_kernel(
 // Segments a wave takes.  One wave per segment (a grid of segments x tokens) is the general
 // shape.  A whole token per wave (a flat grid of tokens, all of the token's loads in flight at
 // once, position and cache row fetched once, every store behind the last rotation) wins where that
-// grid is five to about ten waves per compute unit, which is where a 2048-token chunk plus its
+// grid is five to ten waves per compute unit, which is where a 2048-token chunk plus its
 // decode tokens falls.  Measured on separately allocated tensors, bf16, 32 query + 8 key heads of
 // 128, cold, whole token / one segment per wave: 1024 tokens 5.2 / 5.0 us, 1280 5.8 / 5.8, 1536
-// 6.4 / 6.8, 2048 7.2 / 8.4, 2304 8.1 / 9.3, 2560 9.9 / 10.2, 2816 11.3 / 10.9, 3072 12.2 / 11.6,
-// 4096 16.0 / 14.9 (on inputs still in the memory-side cache the whole token wins throughout).
+// 6.4 / 6.8, 2048 7.2 / 8.4, 2304 8.1 / 9.3, 2560 9.9 / 10.2, 2688 10.7 / 10.5, 2816 11.3 / 10.9,
+// 3072 12.2 / 11.6, 4096 16.0 / 14.9 (on inputs still in the memory-side cache the whole token
+// wins throughout).
 // With 64 query heads (nine segments, i.e. two chunks of five against nine waves of one) 4608
 // tokens take 31.5 against 27.3 us.
 // A wave's loads in flight, not its segment count, are what the limit is about: a NeoX segment is
@@ -293,7 +294,7 @@ struct RopeChunks {
 };
 static RopeChunks plan_rope_chunks(int64_t segs, int64_t tokens, int max_segs) {
   const int64_t units = compute_units();
-  const bool whole_token = segs <= max_segs && tokens >= 5 * units && 2 * tokens <= 21 * units;
+  const bool whole_token = segs <= max_segs && tokens >= 5 * units && 4 * tokens <= 41 * units;
   RopeChunks p;
   p.chunks = whole_token ? 1 : (int)(segs < 1 ? 1 : segs);
   p.spw = whole_token ? (int)(segs < 1 ? 1 : segs) : 1;

@@ -217,6 +217,93 @@ def test_gelu_saturation_and_non_finite_inputs(ops, dev, dtype, name):
     assert_close_dtype(got[mid].reshape(1, -1), want[mid].reshape(1, -1), **_tol(dtype))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("name", ["gelu_new", "gelu_fast"])
+def test_gelu_table_path_every_bit_pattern_same_bits_as_arithmetic_path(ops, dev, dtype, name):
+    """From 12 Mi elements on, 16-bit tensors go through the 65536-entry table in LDS.  A tensor that
+    holds every bit pattern 256 times (shuffled) plus a ragged tail of 5 elements takes that path; the
+    same values in chunks below the threshold take the arithmetic kernel.  Both must give the same
+    bits for every pattern, NaNs, infinities, subnormals and signed zeros included; a sample of the
+    finite values is also checked against the oracle."""
+    op = getattr(ops.activation_ops, name)
+    g = gen(11)
+    pats = torch.arange(65536, dtype=torch.int32).repeat(256)
+    pats = pats[torch.randperm(pats.numel(), generator=g)]
+    pats = torch.cat([pats, torch.tensor([0x3f80, 0xbf80, 0x0001, 0x7fc0, 0x4000], dtype=torch.int32)])
+    x = pats.to(torch.int16).view(dtype).reshape(1, -1).to(dev)            # [1, 2^24 + 5]
+    assert x.numel() == (1 << 24) + 5
+    got = torch.full_like(x, 7.0)
+    op(got, x)                                                               # table path
+    want = torch.full_like(x, 9.0)
+    chunk = 1 << 20
+    for lo in range(0, x.numel(), chunk):                                    # arithmetic path
+        hi = min(lo + chunk, x.numel())
+        piece = torch.empty((1, hi - lo), dtype=dtype, device=dev)
+        op(piece, x[:, lo:hi].contiguous())
+        want[:, lo:hi] = piece
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    # a second call (table complete by now, or still behind its build on this stream) and a call
+    # on another stream give the same bits
+    again = torch.empty_like(x)
+    op(again, x)
+    assert torch.equal(again.view(torch.int16), got.view(torch.int16))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        other = torch.empty_like(x)
+        op(other, x)
+    side.synchronize()
+    assert torch.equal(other.view(torch.int16), got.view(torch.int16))
+    xs = x[:, :4096].cpu()
+    ref = torch.empty_like(xs)
+    getattr(c_oracle, name)(ref, xs)
+    fin = torch.isfinite(ref.float()) & torch.isfinite(xs.float())
+    tol = _tol(dtype)
+    tol["max_mismatch_frac"] = max(tol["max_mismatch_frac"], 2e-2)
+    assert_close_dtype(got[:, :4096].cpu()[fin].reshape(1, -1), ref[fin].reshape(1, -1), **tol)
+
+
+@pytest.mark.parametrize("name", ["gelu_new", "gelu_fast"])
+def test_gelu_table_path_full_size_matches_oracle(ops, dev, name):
+    """[2304, 14336] bf16 (the table path) against the oracle on sampled rows."""
+    g = gen(12)
+    x = randn((2304, 14336), g, torch.bfloat16, std=1.5)
+    got = torch.empty_like(x, device=dev)
+    getattr(ops.activation_ops, name)(got, x.to(dev))
+    rows = torch.randperm(2304, generator=g)[:48]
+    xs = x[rows].contiguous()
+    want = torch.empty_like(xs)
+    getattr(c_oracle, name)(want, xs)
+    tol = _tol(torch.bfloat16)
+    tol["max_mismatch_frac"] = max(tol["max_mismatch_frac"], 2e-2)
+    assert_close_dtype(got.cpu()[rows], want, **tol)
+
+
+def test_gelu_table_path_replayed_in_a_hip_graph(ops, dev):
+    """A large gelu captured into a HIP graph (the table is complete by then: one eager call and a
+    synchronisation first) and replayed on changing inputs gives the eager result every time."""
+    g = gen(13)
+    n = 1 << 24
+    x = randn((1, n), g, torch.bfloat16).to(dev)
+    eager = torch.empty_like(x)
+    ops.activation_ops.gelu_new(eager, x)
+    torch.cuda.synchronize()
+    out = torch.empty_like(x)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            ops.activation_ops.gelu_new(out, x)
+    for rep in range(3):
+        x.copy_(randn((1, n), g, torch.bfloat16))
+        out.fill_(3.0)
+        ops.activation_ops.gelu_new(eager, x)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), rep
+
+
 # ------------------------------------------------------------------ rotary
 
 def _rope_case(ops, dev, dtype, T, nq, nkv, D, R, is_neox, packed, seed=1, prefill=None):

@@ -220,7 +220,7 @@ def test_fused_rope_append_equals_separate_ops(ops, dev, dtype, is_neox, nq, nkv
 ])
 @pytest.mark.parametrize("write_key", [False, True])
 def test_fused_rope_append_one_wave_per_token(ops, dev, nq, nkv, is_neox, write_key):
-    """Batches of 1280..2688 tokens take the kernel shape in which one wave covers a whole token.
+    """Batches of 1280..2624 tokens take the kernel shape in which one wave covers a whole token.
     Checked bit for bit against the two stand-alone ops (each checked against its oracle
     elsewhere), with fewer appended rows than tokens."""
     D, page_size, T, n = 128, 16, 1700, 1650
