@@ -145,9 +145,10 @@ def main():
                     help="moe section: random = N(0,1) router logits (experts get unequal shares, "
                          "as in a real batch); balanced = every expert gets exactly tokens * top_k / "
                          "experts slots (no partly filled slot blocks): shows what the imbalance costs")
-    ap.add_argument("--moe-balance", choices=["on", "off"], default="on",
+    ap.add_argument("--moe-balance", choices=["on", "off"], default="off",
                     help="moe section: spread every expert's slots evenly over its slot blocks before "
-                         "the GEMMs (the library's default) or leave moe_align_block_size's greedy fill")
+                         "the GEMMs (layers.balance_blocks) or leave moe_align_block_size's greedy fill "
+                         "(the library's default)")
     ap.add_argument("--moe-block-m", type=int, default=0,
                     help="moe section: slot-block size of the grouped GEMMs (0 = the library's choice)")
     args = ap.parse_args()

@@ -200,10 +200,10 @@ def test_fused_moe_forward(ops, dev, T, E, k, H, I, renorm):
 @pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("block_m", [64, 128, 256])
 def test_fused_moe_same_bits_with_and_without_balanced_blocks(ops, dev, monkeypatch, packed, block_m):
-    """fused_experts spreads every expert's slots evenly over its blocks before the GEMMs; where a
-    slot sits inside a block does not enter its dot products, so the layer's output is bit for bit
-    the one computed on moe_align_block_size's own layout.  Experts with one, several and no
-    blocks, every block size that is balanced, both weight layouts."""
+    """With BALANCE_BLOCKS set, fused_experts spreads every expert's slots evenly over its blocks
+    before the GEMMs; where a slot sits inside a block does not enter its dot products, so the
+    layer's output is bit for bit the one computed on moe_align_block_size's own layout.  Experts
+    with one, several and no blocks, every block size that is balanced, both weight layouts."""
     import importlib
     fm = importlib.import_module("sarathi_amd.layers.fused_moe")   # the module, not the function
     from sarathi_amd import layers
@@ -219,7 +219,7 @@ def test_fused_moe_same_bits_with_and_without_balanced_blocks(ops, dev, monkeypa
     gating[:, 2] += 1.5                         # and a popular one
     gating = gating.to(dev)
     cfg = {"BLOCK_SIZE_M": block_m, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 64, "GROUP_SIZE_M": 1}
-    assert fm.BALANCE_BLOCKS
+    monkeypatch.setattr(fm, "BALANCE_BLOCKS", True)
     got = layers.fused_moe(x, w1, w2, gating, k, True, override_config=cfg)
     monkeypatch.setattr(fm, "BALANCE_BLOCKS", False)
     want = layers.fused_moe(x, w1, w2, gating, k, True, override_config=cfg)
