@@ -250,6 +250,12 @@ int sarathi_fused_topk_align(float* topk_weights, int32_t* topk_indices,
  * tokens * topk; slots holding a larger id are padding and skipped).
  * block_m must be the block_size moe_align_block_size ran with and one of 32,
  * 64, 128, 256; dtype bf16 or fp16; K a multiple of 64, N a multiple of 4.
+ * dtype fp32 (the reference's fused_experts admits float32 tensors,
+ * fused_moe.py:430) runs a plain float32 matrix-core kernel: row-major weights,
+ * epilogue NONE or ROUTED_WEIGHT, block_m any multiple of 32, K, the strides and
+ * N's pieces multiples of 4; the output is rounded through float16 before it is
+ * stored, as the reference's kernel does with its compute_type for every dtype
+ * but bfloat16 (fused_moe.py:142, 466).
  *
  * b_layout: SARATHI_MOE_B_ROW_MAJOR is the reference's [E, N, K] tensor.
  * SARATHI_MOE_B_PACKED is the same weights re-tiled once, offline, into the

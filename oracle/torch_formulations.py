@@ -132,7 +132,10 @@ def moe_grouped_gemm(A, B, C, topk_weights, sorted_token_ids, expert_ids, num_to
     """What the reference's Triton fused_moe_kernel computes
     (sarathi/model_executor/layers/fused_moe/fused_moe.py:84-147): per block of block_m sorted slots,
     rows A[slot // top_k] times B[expert]^T with fp32 accumulation, optionally times the slot's
-    routing weight (in fp32), cast to the tensor dtype, stored at row `slot` of C."""
+    routing weight (in fp32), cast to the kernel's compute type — bfloat16 for bfloat16 tensors,
+    float16 for everything else, float32 tensors included (fused_moe.py:142, 466) — and stored at
+    row `slot` of C."""
+    compute_type = torch.bfloat16 if C.dtype == torch.bfloat16 else torch.float16
     n_post = int(num_tokens_post_padded.item())
     Cf = C.view(-1, B.shape[1])
     wflat = topk_weights.reshape(-1)
@@ -145,16 +148,18 @@ def moe_grouped_gemm(A, B, C, topk_weights, sorted_token_ids, expert_ids, num_to
         acc = A[slots // top_k].float() @ B[e].float().t()
         if mul_routed_weight:
             acc = acc * wflat[slots].float().unsqueeze(1)
-        Cf[slots] = acc.to(C.dtype)
+        Cf[slots] = acc.to(compute_type).to(C.dtype)
 
 
 def fused_moe(hidden_states, w1, w2, gating_output, topk, renormalize, topk_weights=None,
               topk_ids=None):
     """Dense statement of the MoE layer the reference's fused_moe computes (fused_moe.py:411-622),
     keeping its intermediate tensors in the model dtype: out[t] = sum_j T(w_j * (h_j @ W2[e_j]^T))
-    with h_j = silu_and_mul(T(x_t @ W1[e_j]^T))."""
+    with h_j = silu_and_mul(T(x_t @ W1[e_j]^T)).  T rounds to the kernel's compute type, which is
+    float16 for float32 tensors (fused_moe.py:466)."""
     T, _ = hidden_states.shape
     dt = hidden_states.dtype
+    ct = torch.bfloat16 if dt == torch.bfloat16 else torch.float16
     if topk_ids is not None:      # routing decided by the caller (e.g. grouped_topk)
         tw, ti = topk_weights, topk_ids
     else:
@@ -170,11 +175,11 @@ def fused_moe(hidden_states, w1, w2, gating_output, topk, renormalize, topk_weig
         tok, j = torch.nonzero(ti == e, as_tuple=True)
         if tok.numel() == 0:
             continue
-        gate_up = (hidden_states[tok].float() @ w1[e].float().t()).to(dt)
+        gate_up = (hidden_states[tok].float() @ w1[e].float().t()).to(ct).to(dt)
         act = torch.empty((tok.numel(), inter), dtype=dt)
         silu_and_mul(act, gate_up)
         down = (act.float() @ w2[e].float().t()) * tw[tok, j].unsqueeze(1)
-        parts[tok, j] = down.to(dt)
+        parts[tok, j] = down.to(ct).to(dt)
     return parts.sum(dim=1)
 
 

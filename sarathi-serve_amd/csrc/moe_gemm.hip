@@ -305,6 +305,13 @@ static int launch_moe_gemm(const MoeGemmArgs& g, int epilogue, bool packed, hipS
 // moe_gemm_wide.hip: row-major weights at 64-, 128- and 256-slot blocks, four waves
 int launch_moe_gemm_wide(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, int dtype,
                          hipStream_t st);
+// moe_gemm_f32.hip: float32 tensors
+int launch_moe_gemm_f32(const void* a, const void* b, void* c, const float* topk_weights,
+                        const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                        const int32_t* num_tokens_post_padded, int64_t num_valid_tokens,
+                        int64_t sorted_len, int64_t n, int64_t k, int64_t a_row_stride,
+                        int64_t b_expert_stride, int64_t c_row_stride, int block_m, int top_k,
+                        int epilogue, int b_layout, hipStream_t st);
 
 }  // namespace sarathi_hip
 
@@ -346,6 +353,11 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
     return SARATHI_ERR_INVALID_ARG;
   const bool packed = b_layout == SARATHI_MOE_B_PACKED;
   if (packed && b_expert_stride < (n + 31) / 32 * 32 * k) return SARATHI_ERR_INVALID_ARG;
+  if (dtype == kF32)
+    return launch_moe_gemm_f32(a, b, c, topk_weights, sorted_token_ids, expert_ids,
+                               num_tokens_post_padded, num_valid_tokens, sorted_len, n, k,
+                               a_row_stride, b_expert_stride, c_row_stride, block_m, top_k,
+                               epilogue, b_layout, (hipStream_t)stream);
   if (block_m != 32 && block_m != 64 && block_m != 128 && block_m != 256)
     return SARATHI_ERR_UNSUPPORTED;
   if (dtype != kBF16 && dtype != kF16) return SARATHI_ERR_UNSUPPORTED;

@@ -634,8 +634,11 @@ void moe_grouped_gemm(torch::Tensor& a, torch::Tensor& b, torch::Tensor& c,
   }
   TORCH_CHECK(a.scalar_type() == b.scalar_type() && c.scalar_type() == a.scalar_type(), op,
               ": A, B and C must share a dtype");
-  TORCH_CHECK(a.scalar_type() == at::ScalarType::BFloat16 || a.scalar_type() == at::ScalarType::Half,
-              op, ": only bfloat16 and float16 are supported");
+  TORCH_CHECK(a.scalar_type() == at::ScalarType::BFloat16 || a.scalar_type() == at::ScalarType::Half ||
+                  a.scalar_type() == at::ScalarType::Float,
+              op, ": only bfloat16, float16 and float32 are supported");
+  TORCH_CHECK(a.scalar_type() != at::ScalarType::Float || (!b_packed && !silu_and_mul), op,
+              ": float32 runs on row-major weights without the silu_and_mul epilogue");
   TORCH_CHECK(!(silu_and_mul && mul_routed_weight), op,
               ": silu_and_mul and mul_routed_weight are different epilogues; pick one");
   TORCH_CHECK(!silu_and_mul || n % 2 == 0, op, ": silu_and_mul needs an even N (gate rows, up rows)");

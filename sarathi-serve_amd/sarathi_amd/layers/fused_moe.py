@@ -7,7 +7,10 @@ The two GEMMs are hand-written MFMA kernels (csrc/moe_gemm.hip, csrc/moe_gemm_wi
 the reference's Triton kernel.  Their only free parameter is the slot-block size, which comes from
 the tuned tables under ``configs/`` (the reference's JSON format, written by tune_fused_moe.py)
 when one matches (E, N, device, weight layout), else from ``get_default_config``.
-float16 and bfloat16 only: float32 activations / weights and fp8 weights / scales raise.
+float16 and bfloat16 run the tuned kernels; float32 tensors (which the reference admits,
+fused_moe.py:430) run a plain float32 matrix-core kernel (csrc/moe_gemm_f32.hip) on row-major
+weights, with the reference's rounding of every GEMM output through float16 (fused_moe.py:142, 466);
+fp8 weights / scales raise.
 """
 import functools
 import json
@@ -195,11 +198,14 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
     assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
     assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
     assert w1.is_contiguous() and w2.is_contiguous(), "Expert weights must be contiguous"
-    if hidden_states.dtype not in (torch.float16, torch.bfloat16) or w1.dtype != hidden_states.dtype \
-            or w2.dtype != hidden_states.dtype:
-        raise TypeError("fused_experts runs on the float16 / bfloat16 matrix-core kernels only: got "
-                        f"hidden_states {hidden_states.dtype}, w1 {w1.dtype}, w2 {w2.dtype} (the "
-                        "reference's float32 path has no counterpart here; cast the layer)")
+    if hidden_states.dtype not in (torch.float32, torch.float16, torch.bfloat16) \
+            or w1.dtype != hidden_states.dtype or w2.dtype != hidden_states.dtype:
+        raise TypeError("fused_experts needs float32, float16 or bfloat16 activations and expert weights "
+                        f"of the same dtype: got hidden_states {hidden_states.dtype}, w1 {w1.dtype}, "
+                        f"w2 {w2.dtype}")
+    is_f32 = hidden_states.dtype == torch.float32
+    if is_f32 and (isinstance(w1, PackedExpertWeights) or isinstance(w2, PackedExpertWeights)):
+        raise TypeError("packed expert weights are a 16-bit layout; float32 runs on the [E, N, K] tensors")
     assert w1_scale is None and w2_scale is None and a1_scale is None and a2_scale is None, \
         "fp8 scales are not supported"
     num_tokens, K = hidden_states.shape
@@ -213,7 +219,7 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
         chunk //= 2
     M = min(num_tokens, chunk)
     # gate/up GEMM with the activation fused into its epilogue: no [M, topk, N] intermediate
-    fuse_act = FUSE_SILU_AND_MUL and (N // 2) % 32 == 0
+    fuse_act = FUSE_SILU_AND_MUL and (N // 2) % 32 == 0 and not is_f32
     cache1 = None if fuse_act else torch.empty((M, topk, N), device=dev, dtype=dt)
     cache2 = torch.empty((M * topk, N // 2), device=dev, dtype=dt)
     cache3 = torch.empty((M, topk, w2.shape[1]), device=dev, dtype=dt)

@@ -205,6 +205,9 @@ def test_kv_cache_and_gemm_argument_validation_without_gpu(lib):
     assert gemm(mul=7) == INVALID                   # unknown epilogue code
     assert gemm(mul=2, n=66) == UNSUPPORTED         # gated: N/2 = 33 is not a multiple of 4
     assert gemm(bm=48) == UNSUPPORTED
-    assert gemm(dt=0) == UNSUPPORTED                # fp32 has no matrix-core path here
+    assert gemm(dt=0, layout=1) == UNSUPPORTED      # fp32: row-major weights only,
+    assert gemm(dt=0, mul=2) == UNSUPPORTED         # no gated epilogue,
+    assert gemm(dt=0, bm=48) == UNSUPPORTED         # blocks in multiples of its 32-slot tile
+    assert gemm(dt=7) == UNSUPPORTED
     assert gemm(k=72, astride=72) == UNSUPPORTED    # K must be whole 64-wide steps
     assert gemm(valid=0) == OK

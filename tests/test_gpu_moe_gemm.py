@@ -274,17 +274,82 @@ def test_tuned_config_lookup_and_override(ops, dev):
         layers.get_default_config(512, 7, 1234, 64, 2)
 
 
-def test_fused_experts_rejects_float32(ops, dev):
-    """The reference's Triton kernel also takes float32; the matrix-core kernels here do not, and
-    say so instead of failing inside the launcher."""
+def test_fused_experts_rejects_mixed_dtypes_and_packed_float32(ops, dev):
+    """Activations and both weight tensors must share one of float32 / float16 / bfloat16; the packed
+    layout is a 16-bit one."""
     from sarathi_amd import layers
     x = torch.zeros((4, 64), device=dev)
     w1, w2 = torch.zeros((2, 32, 64), device=dev), torch.zeros((2, 64, 16), device=dev)
     tw, ti = torch.ones((4, 1), device=dev), torch.zeros((4, 1), dtype=torch.int32, device=dev)
-    with pytest.raises(TypeError, match="float16 / bfloat16"):
-        layers.fused_experts(x, w1, w2, tw, ti)
-    with pytest.raises(TypeError, match="float16 / bfloat16"):
+    with pytest.raises(TypeError, match="same dtype"):
         layers.fused_experts(x.half(), w1.half(), w2, tw, ti)
+    with pytest.raises(TypeError, match="same dtype"):
+        layers.fused_experts(x.double(), w1.double(), w2.double(), tw, ti)
+    packed = layers.pack_expert_weights(w1.half())
+    packed.dtype = torch.float32          # a 16-bit packing handed over as if it were float32
+    with pytest.raises(TypeError, match="16-bit layout"):
+        layers.fused_experts(x, packed, w2, tw, ti)
+
+
+@pytest.mark.parametrize("T,E,k,BM,N,K,mul", [
+    (300, 8, 2, 64, 512, 256, False),
+    (300, 8, 2, 64, 512, 256, True),
+    (77, 4, 2, 32, 260, 100, True),      # ragged N, K not a multiple of the 32-deep step
+    (1000, 8, 2, 128, 768, 512, False),
+    (40, 8, 2, 256, 300, 128, False),    # mostly padding
+    (33, 16, 4, 32, 256, 64, True),      # some experts empty
+    (5, 8, 1, 96, 1024, 192, False),     # a block size the 16-bit kernels do not have
+])
+def test_grouped_gemm_float32_matches_formulation(ops, dev, T, E, k, BM, N, K, mul):
+    """float32 tensors: exact float32 products, float32 accumulation, output rounded through
+    float16 as the reference's kernel does for every dtype but bfloat16 (fused_moe.py:142, 466).
+    The accumulation order differs from the CPU matmul's (float32 sums of K products of size ~0.25
+    differ by ~1e-6), so a result may land on the neighbouring float16 value: one float16 ulp of
+    relative tolerance plus 1e-5 absolute, and every stored value must be a float16 value."""
+    _, w, ids, s, e, p = _route(T, E, k, BM, T + N)
+    g = gen(K)
+    A = randn((T, K), g, torch.float32, std=0.5)
+    Bw = randn((E, N, K), g, torch.float32, std=0.5)
+    want = torch.zeros((T, k, N), dtype=torch.float32)
+    torch_formulations.moe_grouped_gemm(A, Bw, want, w, s, e, p, T * k, BM, k, mul)
+    got = torch.full((T, k, N), 7.0, dtype=torch.float32, device=dev)
+    ops.moe_ops.moe_grouped_gemm(A.to(dev), Bw.to(dev), got, w.to(dev), s.to(dev), e.to(dev),
+                                 p.to(dev), T * k, BM, k, mul)
+    got = got.cpu()
+    assert torch.equal(got, got.half().float())
+    assert torch.allclose(got, want, rtol=2 ** -10, atol=1e-5)
+    with pytest.raises(RuntimeError, match="float32"):
+        ops.moe_ops.moe_grouped_gemm(A.to(dev), Bw.to(dev), got.to(dev), w.to(dev), s.to(dev), e.to(dev),
+                                     p.to(dev), T * k, BM, k, False, False, 0, True)
+
+
+def test_grouped_gemm_float32_identity_weights_exact(ops, dev):
+    """One non-zero product per output: the gathered row itself, rounded through float16."""
+    T, E, k, BM, K = 100, 4, 2, 64, 128
+    _, w, ids, s, e, p = _route(T, E, k, BM, 5)
+    A = randn((T, K), gen(6), torch.float32)
+    Bw = torch.eye(K).repeat(E, 1, 1) * torch.arange(1, E + 1, dtype=torch.float32).view(E, 1, 1)
+    got = torch.zeros((T, k, K), dtype=torch.float32, device=dev)
+    ops.moe_ops.moe_grouped_gemm(A.to(dev), Bw.to(dev), got, w.to(dev), s.to(dev), e.to(dev),
+                                 p.to(dev), T * k, BM, k, False)
+    want = (A.unsqueeze(1) * (ids.float() + 1).unsqueeze(-1)).half().float()
+    assert torch.equal(got.cpu(), want)
+
+
+def test_fused_moe_float32_matches_dense_formulation(ops, dev):
+    """The whole layer on float32 tensors (the reference admits them, fused_moe.py:430) against the
+    dense formulation with the same float16 roundings of the two GEMM outputs."""
+    from sarathi_amd import layers
+    T, E, k, H, I = 300, 8, 2, 256, 384
+    g = gen(91)
+    x = randn((T, H), g, torch.float32, std=1.0)
+    w1 = randn((E, 2 * I, H), g, torch.float32, std=H ** -0.5)
+    w2 = randn((E, H, I), g, torch.float32, std=I ** -0.5)
+    gating = torch.randn((T, E), generator=g, dtype=torch.float32)
+    want = torch_formulations.fused_moe(x, w1, w2, gating, k, True)
+    got = layers.fused_moe(x.to(dev), w1.to(dev), w2.to(dev), gating.to(dev), k, True)
+    assert got.dtype == torch.float32
+    assert torch.allclose(got.cpu(), want, rtol=4e-3, atol=4e-3 * want.abs().max().item())
 
 
 @pytest.mark.parametrize("grouped", [False, True])
