@@ -367,6 +367,15 @@ def test_rope_shapes_bit_exact(ops, dev, T, nq, nkv, D, R, is_neox):
         _assert_rope_bits(got, want)
 
 
+@pytest.mark.parametrize("T", [1279, 1280, 2624, 2625])
+def test_rope_launch_shape_boundaries_bit_exact(ops, dev, T):
+    """Either side of the token counts at which the launch switches between one wave per segment and
+    one wave per token (5 and 10.25 waves per compute unit on a 256-unit device), at the Llama-3-8B
+    head counts, packed qkv."""
+    got, want = _rope_case(ops, dev, torch.bfloat16, T, 32, 8, 128, 128, True, True, seed=T)
+    _assert_rope_bits(got, want)
+
+
 @pytest.mark.parametrize("is_neox", [True, False])
 def test_rope_bf16_subnormal_range_and_signed_zeros(ops, dev, is_neox):
     """The bf16 vector path forms each sum of two rounded products with the packed dot-product
