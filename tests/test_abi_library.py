@@ -211,3 +211,38 @@ def test_kv_cache_and_gemm_argument_validation_without_gpu(lib):
     assert gemm(dt=7) == UNSUPPORTED
     assert gemm(k=72, astride=72) == UNSUPPORTED    # K must be whole 64-wide steps
     assert gemm(valid=0) == OK
+
+
+def test_new_entry_points_validate_arguments_without_gpu(lib):
+    """sarathi_moe_gemm_slot_rows is a host-side table; sarathi_moe_balance_blocks and
+    sarathi_stream_copy reject bad sizes before anything is launched."""
+    i64, ci, vp = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p
+    buf = ctypes.create_string_buffer(256)
+    p = ctypes.cast(buf, vp)
+    q = vp(p.value + 128)
+    null = vp(None)
+    INVALID, UNSUPPORTED, OK = -1, -2, 0
+    rows = lib.sarathi_moe_gemm_slot_rows
+    assert [rows(ci(b), ci(0)) for b in (32, 64, 128, 256)] == [1, 2, 2, 2]     # row-major weights
+    assert [rows(ci(b), ci(1)) for b in (32, 64, 128, 256)] == [1, 1, 1, 2]     # packed weights
+    assert rows(ci(48), ci(0)) == UNSUPPORTED and rows(ci(64), ci(7)) == INVALID
+
+    def balance(**kw):
+        return lib.sarathi_moe_balance_blocks(
+            kw.get("src", p), kw.get("dst", q), p, p, i64(kw.get("n", 64)), ci(kw.get("e", 8)),
+            ci(kw.get("b", 64)), ci(64), ci(kw.get("g", 32)), ci(kw.get("r", 1)), null)
+    assert balance(src=null) == INVALID
+    assert balance(dst=p) == INVALID            # in place
+    assert balance(g=0) == INVALID
+    assert balance(r=3) == INVALID              # rows must divide the block
+    assert balance(b=64, r=2, g=64) == INVALID  # granule must divide a row range
+    assert balance(e=2000) == UNSUPPORTED
+    assert balance(n=0) == OK
+
+    def copy(**kw):
+        return lib.sarathi_stream_copy(kw.get("dst", q), kw.get("src", p), i64(kw.get("n", 64)),
+                                       ci(kw.get("kib", 8)), null)
+    assert copy(n=24) == INVALID                # not a multiple of 16 bytes
+    assert copy(dst=vp(q.value + 4)) == INVALID # unaligned
+    assert copy(kib=5) == UNSUPPORTED           # no such launch shape
+    assert copy(n=0) == OK
