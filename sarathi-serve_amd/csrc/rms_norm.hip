@@ -281,14 +281,16 @@ static int launch_rms(void* out, void* in, const void* w, float eps, int64_t T, 
 #define SK_RMS_CASE(WAVES, VPL)                                                               \
   hipLaunchKernelGGL((rms_norm_row_kernel<DT, WAVES, VPL, FUSED>), grid, dim3(64 * WAVES), 0, \
                      st, out, in, w, eps, row_bytes, hidden_f, out_stride * EB, in_stride * EB)
-  // Fused op on rows of 129..512 vectors in mid-sized batches (4 to 12 rows per compute unit): one
-  // wave per row with the stores held back, a grid with no row counts it prefers.  Against the
-  // shapes below at H = 4096 bf16, on separately allocated tensors: 2048 rows 11.9 -> 11.4 us,
-  // 2248 12.9 -> 12.7, 2304 12.9 -> 12.9, 2560 15.8 -> 14.6.  Smaller batches want more waves per
-  // row; from 3072 rows on several rows per wave win (3072: 16.8 against 17.8 us).
+  // Fused op on rows of 129..512 vectors from 4 rows per compute unit on: one wave per row with the
+  // stores held back, a grid with no row counts it prefers.  Against the shapes below, bf16, on
+  // separately allocated tensors, rows of 4096: 2048 rows 11.9 -> 11.4 us, 2560 15.8 -> 14.6,
+  // 3584 21.3 -> 19.5, 4608 27.3 -> 25.8, 8192 46.7 -> 45.2, 32768 181 -> 178 (65536: 370 against 378,
+  // left to the shapes below); rows of 3072 alike; rows of 2048 (four vectors per lane): 4096 rows
+  // 12.4 -> 11.9, 4608 13.8 -> 13.4, but 8192 rows 22.7 against 23.7 and 16384 43.7 against 48.8.
+  // Smaller batches want more waves per row.
   if constexpr (FUSED) {
     const int64_t units = compute_units();
-    if (nvec > 128 && nvec <= 512 && T > 4 * units && T < 12 * units) {
+    if (nvec > 128 && nvec <= 512 && T > 4 * units && T <= (nvec <= 256 ? 24 : 160) * units) {
       if (nvec <= 256)
         hipLaunchKernelGGL((fused_add_rms_norm_wave_kernel<DT, 4>), grid, dim3(64), 0, st, out, in, w,
                            eps, row_bytes, hidden_f, out_stride * EB, in_stride * EB);

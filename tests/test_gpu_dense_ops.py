@@ -62,13 +62,15 @@ def test_fused_add_rms_norm_matches_oracle(ops, dev, dtype, T, H):
     (2304, 3072, torch.bfloat16), (1537, 2560, torch.bfloat16), (2248, 2048, torch.bfloat16),
     (1500, 4096, torch.float16), (1500, 2048, torch.float32), (1100, 1032, torch.float32),
     (3072, 4096, torch.bfloat16), (3073, 4096, torch.bfloat16), (4096, 4096, torch.bfloat16),
-    (4099, 3072, torch.float16)])
+    (4099, 3072, torch.float16), (6144, 2048, torch.bfloat16), (6145, 2048, torch.bfloat16),
+    (40960, 4096, torch.bfloat16), (40963, 4096, torch.bfloat16), (43008, 3072, torch.float16)])
 def test_fused_add_rms_norm_rows_per_workgroup(ops, dev, T, H, dtype):
     """The launch shapes of the fused op on rows of up to 512 vectors: one wave per row with the
-    stores held back (more than 1024 and fewer than 3072 rows: whole and ragged widths, both vector
-    counts per lane, all dtypes), and two or three rows per one-wave workgroup beyond that (3072 ->
-    3, 4096 -> 2, with ragged last workgroups).  Same results as the oracle over every row, through
-    views whose row stride differs from the width."""
+    stores held back (more than 1024 rows, up to 6144 rows of at most 256 vectors or 40960 longer
+    ones: whole and ragged widths, both vector counts per lane, all dtypes), one workgroup per row
+    for more short rows, and two or three rows per one-wave workgroup for more long ones (40963 ->
+    2, 43008 -> 3, with ragged last workgroups).  Same results as the oracle over every row,
+    through views whose row stride differs from the width."""
     g = gen(T + H)
     x, r = randn((T, H), g, dtype), randn((T, H), g, dtype)
     w = randn((H,), g, dtype, mean=1.0, std=0.1)
