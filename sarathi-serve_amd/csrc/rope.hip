@@ -296,9 +296,15 @@ constexpr int kMaxSegsPerWaveGptj = 10;
 struct RopeChunks {
   int chunks, spw;
 };
-static RopeChunks plan_rope_chunks(int64_t segs, int64_t tokens, int max_segs) {
+// With the cache append fused in (the value row's loads and the cache stores ride along), the
+// whole-token shape wins over a wider range, same harness: 1024 tokens 5.5 / 6.5 us, 1536 6.8 / 8.2,
+// 2048 8.3 / 10.2, 2304 9.7 / 11.2, 2560 11.4 / 12.3, 3072 13.5 / 14.3, 4096 17.8 / 18.3; equal at
+// 512 (5.5), behind at 4608 (21.1 / 20.4).
+static RopeChunks plan_rope_chunks(int64_t segs, int64_t tokens, int max_segs, bool append) {
   const int64_t units = compute_units();
-  const bool whole_token = segs <= max_segs && tokens >= 5 * units && 4 * tokens <= 41 * units;
+  const bool in_range = append ? tokens >= 4 * units && tokens <= 16 * units
+                               : tokens >= 5 * units && 4 * tokens <= 41 * units;
+  const bool whole_token = segs <= max_segs && in_range;
   RopeChunks p;
   p.chunks = whole_token ? 1 : (int)(segs < 1 ? 1 : segs);
   p.spw = whole_token ? (int)(segs < 1 ? 1 : segs) : 1;
@@ -379,7 +385,7 @@ static int launch_rope_piece(const RopeLaunch& l, int64_t segs, int64_t num_toke
                              hipStream_t st) {
   if (segs <= 0) return SARATHI_OK;
   const RopeChunks plan =
-      plan_rope_chunks(segs, num_tokens, NEOX ? kMaxSegsPerWave : kMaxSegsPerWaveGptj);
+      plan_rope_chunks(segs, num_tokens, NEOX ? kMaxSegsPerWave : kMaxSegsPerWaveGptj, APPEND);
   const bool flat = plan.chunks == 1;
   const int64_t full_z = flat ? 0 : num_tokens / kMaxGridY;
   const int64_t rem = flat ? num_tokens : num_tokens % kMaxGridY;

@@ -219,11 +219,12 @@ def test_fused_rope_append_equals_separate_ops(ops, dev, dtype, is_neox, nq, nkv
     (24, 8, True),    # four
 ])
 @pytest.mark.parametrize("write_key", [False, True])
-def test_fused_rope_append_one_wave_per_token(ops, dev, nq, nkv, is_neox, write_key):
-    """Batches of 1280..2624 tokens take the kernel shape in which one wave covers a whole token.
-    Checked bit for bit against the two stand-alone ops (each checked against its oracle
-    elsewhere), with fewer appended rows than tokens."""
-    D, page_size, T, n = 128, 16, 1700, 1650
+@pytest.mark.parametrize("T", [1700, 1024, 4096, 4097])
+def test_fused_rope_append_one_wave_per_token(ops, dev, nq, nkv, is_neox, write_key, T):
+    """Batches of 1024..4096 tokens take the kernel shape in which one wave covers a whole token
+    (4097: one wave per segment again).  Checked bit for bit against the two stand-alone ops (each
+    checked against its oracle elsewhere), with fewer appended rows than tokens."""
+    D, page_size, n = 128, 16, T - 50
     g = gen(nq * 100 + nkv)
     pages = (n + page_size - 1) // page_size
     table_pages = torch.randperm(pages + 3, generator=g)[:pages].to(torch.int32).to(dev)
