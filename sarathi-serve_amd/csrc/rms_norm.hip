@@ -322,6 +322,35 @@ static int launch_rms(void* out, void* in, const void* w, float eps, int64_t T, 
     }
 #undef SK_RMS_ROWS
   }
+  // Rows of 513..1024 vectors (hidden sizes 4104..8192 in 16-bit types), 4 rows per compute unit
+  // and up: one wave per row (10..16 vectors per lane) for as long as every wave of the launch is
+  // resident at once, so that the launch is one read phase followed by one write phase.  bf16, cold,
+  // separately allocated tensors, multi-wave shape below -> one wave; plain norm: rows of 5120,
+  // 1024 rows 5.5 -> 4.9 us, 2304 10.0 -> 8.8, 4096 15.6 -> 14.8 (4608: 17.5 against 19.3); rows of
+  // 7168, 2304 rows 13.1 -> 11.4, 3072 16.4 -> 15.2 (3584: 18.9 against 21.2); rows of 8192, 2048
+  // rows 13.3 -> 11.3, 3072 18.5 -> 17.2 (3584: 21.0 against 23.7).  Fused op (stores held back):
+  // rows of 5120, 2304 rows 16.8 -> 15.3, 3072 21.5 -> 20.0 (3584: 24.8 against 25.8); rows of
+  // 7168, 2048 rows 20.5 -> 18.6 (2560 equal, 3072 behind); rows of 8192, 2048 rows 22.8 -> 20.9
+  // (2560: 27.8 against 28.3).  Below 4 rows per unit the multi-wave shapes are ahead.
+  if (nvec > 512 && nvec <= 1024) {
+    const int64_t units = compute_units();
+    const int vpl = 2 * ((nvec + 127) / 128);  // 10, 12, 14 or 16
+    const int64_t cap = FUSED ? (vpl == 10 ? 12 : 8) : (vpl <= 12 ? 16 : 12);
+    if (T >= 4 * units && T <= cap * units) {
+#define SK_RMS_WAVE(VPL)                                                                         \
+  case VPL:                                                                                      \
+    if constexpr (FUSED)                                                                         \
+      hipLaunchKernelGGL((fused_add_rms_norm_wave_kernel<DT, VPL>), grid, dim3(64), 0, st, out,  \
+                         in, w, eps, row_bytes, hidden_f, out_stride * EB, in_stride * EB);      \
+    else                                                                                         \
+      SK_RMS_CASE(1, VPL);                                                                       \
+    return launch_status();
+      switch (vpl) {
+        SK_RMS_WAVE(10) SK_RMS_WAVE(12) SK_RMS_WAVE(14) SK_RMS_WAVE(16)
+      }
+#undef SK_RMS_WAVE
+    }
+  }
   // One row per workgroup.  Shapes measured on MI355X at H = 4096 and H = 8192 (bf16).  The plain
   // norm is fastest with a whole row of up to 512 vectors in ONE wave (no LDS, no barrier) and
   // four vectors per lane beyond that; the fused op, which holds two rows' worth of loads, is

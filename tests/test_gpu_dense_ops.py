@@ -58,6 +58,44 @@ def test_fused_add_rms_norm_matches_oracle(ops, dev, dtype, T, H):
 
 
 @pytest.mark.parametrize("T,H,dtype", [
+    (1100, 5120, torch.bfloat16), (1024, 4544, torch.bfloat16), (1500, 6144, torch.float16),
+    (1300, 7168, torch.bfloat16), (2048, 8192, torch.bfloat16), (2049, 8192, torch.bfloat16),
+    (1100, 4104, torch.float16), (1200, 3000, torch.float32), (1200, 4096, torch.float32),
+    (3072, 5120, torch.bfloat16), (3073, 5120, torch.bfloat16), (4096, 5120, torch.bfloat16),
+    (4097, 5120, torch.bfloat16), (3073, 8192, torch.float16)])
+def test_rms_norm_long_rows_one_wave_per_row(ops, dev, T, H, dtype):
+    """Rows of 513..1024 sixteen-byte vectors from four rows per compute unit on: one wave per
+    row with 10, 12, 14 or 16 vectors per lane (whole and ragged widths), for both ops, up to the
+    row counts where each hands over to the multi-wave shapes (one row below and above).  Same
+    results as the oracle through views whose row stride differs from the width."""
+    g = gen(T + H)
+    x, r = randn((T, H), g, dtype), randn((T, H), g, dtype)
+    w = randn((H,), g, dtype, mean=1.0, std=0.1)
+    pad = 64
+    # plain norm
+    want = torch.empty_like(x)
+    c_oracle.rms_norm(want, x, w, 1e-5)
+    in_buf = torch.zeros((T, H + pad), dtype=dtype, device=dev)
+    out_buf = torch.zeros((T, H + 2 * pad), dtype=dtype, device=dev)
+    in_buf[:, :H].copy_(x)
+    ops.layernorm_ops.rms_norm(out_buf[:, :H], in_buf[:, :H], w.to(dev), 1e-5)
+    assert_close_dtype(out_buf[:, :H], want, **_tol(dtype))
+    assert bool((out_buf[:, H:] == 0).all())
+    # fused op
+    wx, wr = x.clone(), r.clone()
+    c_oracle.fused_add_rms_norm(wx, wr, w, 1e-5)
+    gx_buf = torch.zeros((T, H + pad), dtype=dtype, device=dev)
+    gr_buf = torch.zeros((T, H + 8), dtype=dtype, device=dev)
+    gx, gr = gx_buf[:, :H], gr_buf[:, :H]
+    gx.copy_(x)
+    gr.copy_(r)
+    ops.layernorm_ops.fused_add_rms_norm(gx, gr, w.to(dev), 1e-5)
+    assert torch.equal(gr.cpu(), wr), "residual = T(x + r) must be bit-exact"
+    assert_close_dtype(gx, wx, **_tol(dtype))
+    assert bool((gx_buf[:, H:] == 0).all()) and bool((gr_buf[:, H:] == 0).all())
+
+
+@pytest.mark.parametrize("T,H,dtype", [
     (2304, 4096, torch.bfloat16), (2305, 4096, torch.bfloat16), (1030, 4096, torch.bfloat16),
     (2304, 3072, torch.bfloat16), (1537, 2560, torch.bfloat16), (2248, 2048, torch.bfloat16),
     (1500, 4096, torch.float16), (1500, 2048, torch.float32), (1100, 1032, torch.float32),
