@@ -103,6 +103,30 @@ SK_DEV void rotate_slot(u32x4& xr, u32x4& yr, const Vec<DT>& c, const Vec<DT>& s
   }
 }
 
+// Heads of 128 bytes (NeoX, head_size 64 in a 16-bit type, fully rotated): the x half and the y
+// half of a head share one 128-byte line, and a load that takes the x vectors of 16 heads touches
+// half of each of 16 lines, the y load the other halves.  The paired layout reads memory in order
+// instead: eight consecutive lanes take the eight 16-byte pieces of one head (x x x x y y y y),
+// the wave's first load the first eight heads of the segment and the second load the next eight,
+// each 1 KiB of consecutive bytes.  A lane then holds the same piece of two heads; the lanes of a
+// head's x pieces trade their second register for the first register of the lane four up, after
+// which every lane holds an x vector and the matching y vector of ONE head (lanes 0-3 of a group
+// of eight the first load's head, lanes 4-7 the second load's), exactly what rotate_slot() takes.
+// The same trade after the rotation puts the results back in memory order.  Two DPP moves per
+// dword, bank-masked so that each direction writes only its receivers.
+SK_DEV void trade_pairs(u32x4& lo, u32x4& hi) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int a = (int)lo[i], b = (int)hi[i];
+    // lanes 0-3 and 8-11 of each row of 16: hi <- lo of the lane four up (row_shl:4)
+    const int nb = __builtin_amdgcn_update_dpp(b, a, 0x104, 0xf, 0x5, false);
+    // lanes 4-7 and 12-15: lo <- hi of the lane four down (row_shr:4)
+    const int na = __builtin_amdgcn_update_dpp(a, b, 0x114, 0xf, 0xa, false);
+    lo[i] = (uint32_t)na;
+    hi[i] = (uint32_t)nb;
+  }
+}
+
 // Store policy of the in-place results.  With a wave per token the rows it rewrites are still in
 // L2 from its own loads; a non-temporal write-back store measured 2 % faster there than the
 // write-through store that wins for out-of-place streams and for the one-segment shape.
@@ -145,7 +169,7 @@ constexpr uint32_t kRopeAIsKey = 0x80000000u;
 // rot_dim == head_size, which this path requires, the x and y vectors of a k segment cover its
 // heads completely, so the v vectors at the same two offsets cover the same heads of the v row.
 // The entry address is resolved with scalar loads while the data loads are in flight.
-template <int DT, bool NEOX, int SPW, bool FLAT, bool APPEND>
+template <int DT, bool NEOX, int SPW, bool FLAT, bool APPEND, bool PAIRED>
 SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
                       const void* __restrict__ cache, int64_t a_stride_bytes, int64_t delta0,
                       int64_t delta_step, uint32_t geom, uint32_t heads,
@@ -164,26 +188,39 @@ SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
   const rsrc_t r = make_rsrc(reinterpret_cast<char*>(a) + tok * a_stride_bytes, 0x7fffffffu);
   const uint32_t a_pad = (((heads_a << sh) + 63u) >> 6) << (6 - sh);  // A's heads in whole segments
   const uint32_t slot = threadIdx.x & ((1u << sh) - 1u);
-  const uint32_t h0 = chunk * (uint32_t)(SPW << (6 - sh)) + (threadIdx.x >> sh);
+  // PAIRED (sh == 2): the lane's piece of its head in memory order, see trade_pairs()
+  const uint32_t h0 = chunk * (uint32_t)(SPW << (6 - sh)) + (threadIdx.x >> (PAIRED ? 3 : sh));
+  const uint32_t piece = PAIRED ? (threadIdx.x & 7u) * 16u : slot * 16u;
 
   const uint32_t kv_row_bytes = (a_is_key ? heads_a : heads_b) * head_bytes;
 
   u32x4 xr[SPW], yr[SPW], vx[SPW], vy[SPW];
-  uint32_t xoff[SPW];   // offset of the lane's x vector from A's row
+  uint32_t xoff[SPW];   // offset of the lane's first vector (x) from A's row
   uint32_t koff[SPW];   // APPEND: the same offset inside the k / v row
+  uint32_t yoff[SPW], kyoff[SPW];  // the second vector: y of the same head; PAIRED: eight heads on
+  // where a head's piece lies: from A's row (query / key traffic) and inside its own row
+  auto locate = [&](uint32_t h, uint32_t& from_a, uint32_t& in_row) {
+    const uint32_t hb = h - a_pad;  // wraps to a huge value while h is inside A's padded span
+    const bool in_a = h < heads_a, in_b = hb < heads_b;
+    const uint32_t row_off = (in_a ? h : hb) * head_bytes + piece;
+    from_a = (in_a || in_b) ? row_off + (in_a ? 0u : delta) : kClipped;
+    in_row = (in_a || in_b) ? row_off : kClipped;
+  };
   // The query / key loads need nothing beyond the kernel arguments that the hardware preloads into
   // scalar registers (the first 14 dwords), so they leave before the wave has waited for anything;
   // the value loads and the append bookkeeping read later arguments and follow them.
 #pragma unroll
   for (int j = 0; j < SPW; ++j) {
     const uint32_t h = h0 + (uint32_t)(j << (6 - sh));
-    const uint32_t hb = h - a_pad;  // wraps to a huge value while h is inside A's padded span
-    const bool in_a = h < heads_a, in_b = hb < heads_b;
-    const uint32_t row_off = (in_a ? h : hb) * head_bytes + slot * 16u;
-    xoff[j] = (in_a || in_b) ? row_off + (in_a ? 0u : delta) : kClipped;
-    koff[j] = (in_a || in_b) ? row_off : kClipped;
+    locate(h, xoff[j], koff[j]);
+    if constexpr (PAIRED) {
+      locate(h + 8u, yoff[j], kyoff[j]);
+    } else {
+      yoff[j] = xoff[j] + embed_bytes;
+      kyoff[j] = koff[j] + embed_bytes;
+    }
     xr[j] = buf_load16<kStreamLoad>(r, xoff[j]);
-    if constexpr (NEOX) yr[j] = buf_load16<kStreamLoad>(r, xoff[j] + embed_bytes);
+    if constexpr (NEOX) yr[j] = buf_load16<kStreamLoad>(r, yoff[j]);
   }
   bool appended = false;
   if constexpr (APPEND) {
@@ -198,7 +235,7 @@ SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
         const rsrc_t rv = make_rsrc(
             reinterpret_cast<const char*>(value) + tok * v_stride_bytes, kv_row_bytes);
         vx[j] = buf_load16<kStreamLoad>(rv, koff[j]);
-        if constexpr (NEOX) vy[j] = buf_load16<kStreamLoad>(rv, koff[j] + embed_bytes);
+        if constexpr (NEOX) vy[j] = buf_load16<kStreamLoad>(rv, kyoff[j]);
       }
     }
   }
@@ -232,7 +269,11 @@ SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
   // reads down.  2048-2560 tokens of 32 + 8 heads: 7-9 % faster (2304: 8.2 -> 7.6 us); within 4 %
   // either way at 1536 and 3072 tokens.
 #pragma unroll
-  for (int j = 0; j < SPW; ++j) rotate_slot<DT, NEOX>(xr[j], yr[j], c, s);
+  for (int j = 0; j < SPW; ++j) {
+    if constexpr (PAIRED) trade_pairs(xr[j], yr[j]);
+    rotate_slot<DT, NEOX>(xr[j], yr[j], c, s);
+    if constexpr (PAIRED) trade_pairs(xr[j], yr[j]);
+  }
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int j = 0; j < SPW; ++j) {
@@ -245,33 +286,34 @@ SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
         const rsrc_t rkc = make_rsrc(reinterpret_cast<char*>(d->k_cache) + entry, kv_row_bytes);
         const rsrc_t rvc = make_rsrc(reinterpret_cast<char*>(d->v_cache) + entry, kv_row_bytes);
         buf_store16<kKvStoreFused>(rkc, koff[j], xr[j]);
-        if constexpr (NEOX) buf_store16<kKvStoreFused>(rkc, koff[j] + embed_bytes, yr[j]);
+        if constexpr (NEOX) buf_store16<kKvStoreFused>(rkc, kyoff[j], yr[j]);
         buf_store16<kKvStoreFused>(rvc, koff[j], vx[j]);
-        if constexpr (NEOX) buf_store16<kKvStoreFused>(rvc, koff[j] + embed_bytes, vy[j]);
+        if constexpr (NEOX) buf_store16<kKvStoreFused>(rvc, kyoff[j], vy[j]);
       }
     }
     if (in_place) {
       buf_store16<SP>(r, xoff[j], xr[j]);
-      if constexpr (NEOX) buf_store16<SP>(r, xoff[j] + embed_bytes, yr[j]);
+      if constexpr (NEOX) buf_store16<SP>(r, yoff[j], yr[j]);
     }
   }
 }
 
-template <int DT, bool NEOX, int SPW, bool FLAT>
+template <int DT, bool NEOX, int SPW, bool FLAT, bool PAIRED>
 __global__ __launch_bounds__(64) void rope_tok_kernel(
     const int64_t* __restrict__ positions, void* a, const void* __restrict__ cache,
     int64_t a_stride_bytes, int64_t delta0, int64_t delta_step, uint32_t geom, uint32_t heads) {
-  rope_wave<DT, NEOX, SPW, FLAT, false>(positions, a, cache, a_stride_bytes, delta0, delta_step,
-                                        geom, heads, nullptr, 0, 0, nullptr);
+  rope_wave<DT, NEOX, SPW, FLAT, false, PAIRED>(positions, a, cache, a_stride_bytes, delta0,
+                                                delta_step, geom, heads, nullptr, 0, 0, nullptr);
 }
 
-template <int DT, bool NEOX, int SPW, bool FLAT>
+template <int DT, bool NEOX, int SPW, bool FLAT, bool PAIRED>
 __global__ __launch_bounds__(64) void rope_append_tok_kernel(
     const int64_t* __restrict__ positions, void* a, const void* __restrict__ cache,
     int64_t a_stride_bytes, int64_t delta0, int64_t delta_step, uint32_t geom, uint32_t heads,
     const void* __restrict__ value, int64_t v_stride_bytes, uint32_t write_key, KvDest d) {
-  rope_wave<DT, NEOX, SPW, FLAT, true>(positions, a, cache, a_stride_bytes, delta0, delta_step,
-                                       geom, heads, value, v_stride_bytes, write_key, &d);
+  rope_wave<DT, NEOX, SPW, FLAT, true, PAIRED>(positions, a, cache, a_stride_bytes, delta0,
+                                               delta_step, geom, heads, value, v_stride_bytes,
+                                               write_key, &d);
 }
 
 // Segments a wave takes.  One wave per segment (a grid of segments x tokens) is the general
@@ -412,16 +454,28 @@ static int launch_rope_piece(const RopeLaunch& l, int64_t segs, int64_t num_toke
   const dim3 block(64);
   const dim3 grid_full((unsigned)plan.chunks, kMaxGridY, (unsigned)full_z);
   const dim3 grid_rem = flat ? dim3((unsigned)rem) : dim3((unsigned)plan.chunks, (unsigned)rem, 1);
-#define SK_ROPE_GO(SPW, FLAT, GRID, L, VALUE, DEST)                                              \
+  // heads of 128 bytes, fully rotated: memory-order loads (trade_pairs)
+  const bool paired = NEOX && (l.geom & 0xffffu) == 128u && (l.geom >> 16) == 64u;
+#define SK_ROPE_GO1(SPW, FLAT, PAIRED, GRID, L, VALUE, DEST)                                     \
   do {                                                                                           \
     if constexpr (APPEND)                                                                        \
-      hipLaunchKernelGGL((rope_append_tok_kernel<DT, NEOX, SPW, FLAT>), GRID, block, 0, st,      \
-                         L.positions, L.a, L.cache, L.a_stride_bytes, L.delta0, L.delta_step,    \
-                         L.geom, L.heads, VALUE, vsb, (uint32_t)write_key, DEST);                \
+      hipLaunchKernelGGL((rope_append_tok_kernel<DT, NEOX, SPW, FLAT, PAIRED>), GRID, block, 0,  \
+                         st, L.positions, L.a, L.cache, L.a_stride_bytes, L.delta0,              \
+                         L.delta_step, L.geom, L.heads, VALUE, vsb, (uint32_t)write_key, DEST);  \
     else                                                                                         \
-      hipLaunchKernelGGL((rope_tok_kernel<DT, NEOX, SPW, FLAT>), GRID, block, 0, st,             \
+      hipLaunchKernelGGL((rope_tok_kernel<DT, NEOX, SPW, FLAT, PAIRED>), GRID, block, 0, st,     \
                          L.positions, L.a, L.cache, L.a_stride_bytes, L.delta0, L.delta_step,    \
                          L.geom, L.heads);                                                       \
+  } while (0)
+#define SK_ROPE_GO(SPW, FLAT, GRID, L, VALUE, DEST)                                              \
+  do {                                                                                           \
+    if constexpr (NEOX) {                                                                        \
+      if (paired) {                                                                              \
+        SK_ROPE_GO1(SPW, FLAT, true, GRID, L, VALUE, DEST);                                      \
+        break;                                                                                   \
+      }                                                                                          \
+    }                                                                                            \
+    SK_ROPE_GO1(SPW, FLAT, false, GRID, L, VALUE, DEST);                                         \
   } while (0)
 #define SK_ROPE_LAUNCH(SPW)                                                \
   case SPW:                                                                \
@@ -446,6 +500,7 @@ static int launch_rope_piece(const RopeLaunch& l, int64_t segs, int64_t num_toke
   }
 #undef SK_ROPE_LAUNCH
 #undef SK_ROPE_GO
+#undef SK_ROPE_GO1
   return launch_status();
 }
 

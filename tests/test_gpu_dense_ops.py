@@ -407,6 +407,24 @@ def test_rope_shapes_bit_exact(ops, dev, T, nq, nkv, D, R, is_neox):
         _assert_rope_bits(got, want)
 
 
+@pytest.mark.parametrize("dtype,D", [(torch.bfloat16, 64), (torch.float16, 64), (torch.float32, 32)])
+@pytest.mark.parametrize("T,nq,nkv", [
+    (37, 71, 1),       # Falcon-7B: 71 query heads and one key head, one wave per segment
+    (1700, 71, 1),     # six segments: still one wave per segment
+    (1700, 40, 8),     # three segments: one wave per token
+    (1500, 9, 9),      # nine heads in segments of sixteen, one wave per token
+    (300, 128, 8),     # Falcon-40B
+    (2304, 16, 16),    # whole segments only
+])
+def test_rope_neox_heads_of_128_bytes_bit_exact(ops, dev, dtype, D, T, nq, nkv):
+    """NeoX heads of 128 bytes (head_size 64 in a 16-bit type, 32 in float32), fully rotated: the
+    kernels read them in memory order, eight lanes per head, and lanes trade registers before and
+    after the rotation.  Same bits as the oracle, contiguous and packed qkv."""
+    for packed in (False, True):
+        got, want = _rope_case(ops, dev, dtype, T, nq, nkv, D, D, True, packed, seed=T + nq)
+        _assert_rope_bits(got, want)
+
+
 @pytest.mark.parametrize("T", [1279, 1280, 2624, 2625])
 def test_rope_launch_shape_boundaries_bit_exact(ops, dev, T):
     """Either side of the token counts at which the launch switches between one wave per segment and

@@ -211,20 +211,23 @@ def test_fused_rope_append_equals_separate_ops(ops, dev, dtype, is_neox, nq, nkv
         assert np.array_equal(_bits(ok[:n]), _bits(untouched[:n]))
 
 
-@pytest.mark.parametrize("nq,nkv,is_neox", [
-    (32, 8, False),   # ten segments of interleaved pairs in one wave
-    (28, 8, False),   # nine
-    (20, 4, False),   # six
-    (12, 4, True),    # two NeoX segments
-    (24, 8, True),    # four
+@pytest.mark.parametrize("nq,nkv,is_neox,D", [
+    (32, 8, False, 128),   # ten segments of interleaved pairs in one wave
+    (28, 8, False, 128),   # nine
+    (20, 4, False, 128),   # six
+    (12, 4, True, 128),    # two NeoX segments
+    (24, 8, True, 128),    # four
+    (71, 1, True, 64),     # heads of 128 bytes (memory-order loads): Falcon-7B, five q segments + one
+    (40, 8, True, 64),     # three segments, the key heads in the first half of theirs
+    (9, 9, True, 64),      # ragged: nine heads in a segment of sixteen, for q and for k
 ])
 @pytest.mark.parametrize("write_key", [False, True])
 @pytest.mark.parametrize("T", [1700, 1024, 4096, 4097])
-def test_fused_rope_append_one_wave_per_token(ops, dev, nq, nkv, is_neox, write_key, T):
+def test_fused_rope_append_one_wave_per_token(ops, dev, nq, nkv, is_neox, D, write_key, T):
     """Batches of 1024..4096 tokens take the kernel shape in which one wave covers a whole token
     (4097: one wave per segment again).  Checked bit for bit against the two stand-alone ops (each
     checked against its oracle elsewhere), with fewer appended rows than tokens."""
-    D, page_size, n = 128, 16, T - 50
+    page_size, n = 16, T - 50
     g = gen(nq * 100 + nkv)
     pages = (n + page_size - 1) // page_size
     table_pages = torch.randperm(pages + 3, generator=g)[:pages].to(torch.int32).to(dev)
