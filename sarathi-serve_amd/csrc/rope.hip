@@ -190,14 +190,24 @@ SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
   const uint32_t slot = threadIdx.x & ((1u << sh) - 1u);
   // PAIRED (sh == 2): the lane's piece of its head in memory order, see trade_pairs()
   const uint32_t h0 = chunk * (uint32_t)(SPW << (6 - sh)) + (threadIdx.x >> (PAIRED ? 3 : sh));
-  const uint32_t piece = PAIRED ? (threadIdx.x & 7u) * 16u : slot * 16u;
+  const uint32_t piece = (threadIdx.x & 7u) * 16u;  // PAIRED only
 
   const uint32_t kv_row_bytes = (a_is_key ? heads_a : heads_b) * head_bytes;
 
   u32x4 xr[SPW], yr[SPW], vx[SPW], vy[SPW];
   uint32_t xoff[SPW];   // offset of the lane's first vector (x) from A's row
   uint32_t koff[SPW];   // APPEND: the same offset inside the k / v row
-  uint32_t yoff[SPW], kyoff[SPW];  // the second vector: y of the same head; PAIRED: eight heads on
+  // The second vector of a lane: the y vector of the same head, embed_bytes on; PAIRED: the same
+  // piece of the head eight heads on, at offsets of its own.
+  uint32_t yoff2[PAIRED ? SPW : 1], kyoff2[PAIRED ? SPW : 1];
+  auto yoff = [&](int j) -> uint32_t {
+    if constexpr (PAIRED) return yoff2[j];
+    else return xoff[j] + embed_bytes;
+  };
+  auto kyoff = [&](int j) -> uint32_t {
+    if constexpr (PAIRED) return kyoff2[j];
+    else return koff[j] + embed_bytes;
+  };
   // where a head's piece lies: from A's row (query / key traffic) and inside its own row
   auto locate = [&](uint32_t h, uint32_t& from_a, uint32_t& in_row) {
     const uint32_t hb = h - a_pad;  // wraps to a huge value while h is inside A's padded span
@@ -212,15 +222,18 @@ SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
 #pragma unroll
   for (int j = 0; j < SPW; ++j) {
     const uint32_t h = h0 + (uint32_t)(j << (6 - sh));
-    locate(h, xoff[j], koff[j]);
     if constexpr (PAIRED) {
-      locate(h + 8u, yoff[j], kyoff[j]);
+      locate(h, xoff[j], koff[j]);
+      locate(h + 8u, yoff2[j], kyoff2[j]);
     } else {
-      yoff[j] = xoff[j] + embed_bytes;
-      kyoff[j] = koff[j] + embed_bytes;
+      const uint32_t hb = h - a_pad;  // wraps to a huge value while h is inside A's padded span
+      const bool in_a = h < heads_a, in_b = hb < heads_b;
+      const uint32_t row_off = (in_a ? h : hb) * head_bytes + slot * 16u;
+      xoff[j] = (in_a || in_b) ? row_off + (in_a ? 0u : delta) : kClipped;
+      koff[j] = (in_a || in_b) ? row_off : kClipped;
     }
     xr[j] = buf_load16<kStreamLoad>(r, xoff[j]);
-    if constexpr (NEOX) yr[j] = buf_load16<kStreamLoad>(r, yoff[j]);
+    if constexpr (NEOX) yr[j] = buf_load16<kStreamLoad>(r, yoff(j));
   }
   bool appended = false;
   if constexpr (APPEND) {
@@ -235,7 +248,7 @@ SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
         const rsrc_t rv = make_rsrc(
             reinterpret_cast<const char*>(value) + tok * v_stride_bytes, kv_row_bytes);
         vx[j] = buf_load16<kStreamLoad>(rv, koff[j]);
-        if constexpr (NEOX) vy[j] = buf_load16<kStreamLoad>(rv, kyoff[j]);
+        if constexpr (NEOX) vy[j] = buf_load16<kStreamLoad>(rv, kyoff(j));
       }
     }
   }
@@ -286,14 +299,14 @@ SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
         const rsrc_t rkc = make_rsrc(reinterpret_cast<char*>(d->k_cache) + entry, kv_row_bytes);
         const rsrc_t rvc = make_rsrc(reinterpret_cast<char*>(d->v_cache) + entry, kv_row_bytes);
         buf_store16<kKvStoreFused>(rkc, koff[j], xr[j]);
-        if constexpr (NEOX) buf_store16<kKvStoreFused>(rkc, kyoff[j], yr[j]);
+        if constexpr (NEOX) buf_store16<kKvStoreFused>(rkc, kyoff(j), yr[j]);
         buf_store16<kKvStoreFused>(rvc, koff[j], vx[j]);
-        if constexpr (NEOX) buf_store16<kKvStoreFused>(rvc, kyoff[j], vy[j]);
+        if constexpr (NEOX) buf_store16<kKvStoreFused>(rvc, kyoff(j), vy[j]);
       }
     }
     if (in_place) {
       buf_store16<SP>(r, xoff[j], xr[j]);
-      if constexpr (NEOX) buf_store16<SP>(r, yoff[j], yr[j]);
+      if constexpr (NEOX) buf_store16<SP>(r, yoff(j), yr[j]);
     }
   }
 }
@@ -342,14 +355,41 @@ struct RopeChunks {
 // whole-token shape wins over a wider range, same harness: 1024 tokens 5.5 / 6.5 us, 1536 6.8 / 8.2,
 // 2048 8.3 / 10.2, 2304 9.7 / 11.2, 2560 11.4 / 12.3, 3072 13.5 / 14.3, 4096 17.8 / 18.3; equal at
 // 512 (5.5), behind at 4608 (21.1 / 20.4).
-static RopeChunks plan_rope_chunks(int64_t segs, int64_t tokens, int max_segs, bool append) {
+//
+// Tokens of more than max_segs segments (64 query heads of 128, or as many key heads as query
+// heads) can be dealt to a few waves of up to max_segs segments each, in equal parts where the
+// count allows (nine segments as 3 x 3, eight as 2 x 4).  That wins in the same place, four to
+// eight such waves per compute unit, i.e. at 500-1000 tokens; bf16, cold, one wave per segment ->
+// dealt: 32 + 32 heads, 768 tokens 5.9 -> 5.1 us, 1024 7.2 -> 6.4 (1280 equal); 40 + 40 heads, 640
+// tokens 6.0 -> 5.4, 1024 8.5 -> 8.0 (1152: 9.4 against 9.9); 64 + 8 heads, 512 tokens 4.8 -> 4.5,
+// 768 6.1 -> 5.7 (896: 7.0 against 7.2); 64 + 64 heads, 512 tokens 7.2 -> 6.4 (640 equal).  With
+// the append fused in the gain ends earlier, at five waves per unit (40 + 40 heads, 640 tokens
+// 8.9 -> 8.6, 768 10.4 against 10.5; 32 + 32 heads, 768 tokens 9.4 -> 8.1, 1024 equal), unless
+// the key heads are a small part of the token: 56 + 8 heads gain at every size measured (1024
+// tokens 10.1 -> 7.7 us, 1536 14.1 -> 12.0), 64 + 8 heads up to nine waves per unit.
+static RopeChunks plan_rope_chunks(int64_t segs, int64_t key_segs, int64_t tokens, int max_segs,
+                                   bool append) {
   const int64_t units = compute_units();
-  const bool in_range = append ? tokens >= 4 * units && tokens <= 16 * units
-                               : tokens >= 5 * units && 4 * tokens <= 41 * units;
-  const bool whole_token = segs <= max_segs && in_range;
   RopeChunks p;
-  p.chunks = whole_token ? 1 : (int)(segs < 1 ? 1 : segs);
-  p.spw = whole_token ? (int)(segs < 1 ? 1 : segs) : 1;
+  p.chunks = (int)(segs < 1 ? 1 : segs);
+  p.spw = 1;
+  if (segs <= max_segs) {
+    const bool in_range = append ? tokens >= 4 * units && tokens <= 16 * units
+                                 : tokens >= 5 * units && 4 * tokens <= 41 * units;
+    if (in_range) {
+      p.chunks = 1;
+      p.spw = (int)(segs < 1 ? 1 : segs);
+    }
+    return p;
+  }
+  int64_t parts = (segs + max_segs - 1) / max_segs;
+  if (segs % parts != 0 && segs % (parts + 1) == 0) ++parts;
+  const int64_t waves = parts * tokens;
+  const int64_t lo = append ? 3 : 4, hi = append && 4 * key_segs > segs ? 5 : 8;
+  if (waves >= lo * units && waves <= hi * units) {
+    p.chunks = (int)parts;
+    p.spw = (int)((segs + parts - 1) / parts);
+  }
   return p;
 }
 
@@ -426,8 +466,11 @@ static int launch_rope_piece(const RopeLaunch& l, int64_t segs, int64_t num_toke
                              const void* value, int64_t vsb, int write_key, const KvDest* d,
                              hipStream_t st) {
   if (segs <= 0) return SARATHI_OK;
+  const uint32_t sh = (l.heads >> 24) & 0x7fu;
+  const int64_t key_heads = (l.heads & kRopeAIsKey) ? (l.heads & 0xfffu) : ((l.heads >> 12) & 0xfffu);
   const RopeChunks plan =
-      plan_rope_chunks(segs, num_tokens, NEOX ? kMaxSegsPerWave : kMaxSegsPerWaveGptj, APPEND);
+      plan_rope_chunks(segs, ((key_heads << sh) + 63) >> 6, num_tokens,
+                       NEOX ? kMaxSegsPerWave : kMaxSegsPerWaveGptj, APPEND);
   const bool flat = plan.chunks == 1;
   const int64_t full_z = flat ? 0 : num_tokens / kMaxGridY;
   const int64_t rem = flat ? num_tokens : num_tokens % kMaxGridY;

@@ -400,6 +400,10 @@ def test_rope_llama3_8b_hybrid_batch_bit_exact(ops, dev, dtype, is_neox, packed)
     (1700, 20, 4, 128, 128),        # one wave per token: 3 NeoX segments / 6 of interleaved pairs
     (1700, 28, 8, 128, 128),        # 5 / 9 segments
     (1600, 44, 4, 128, 128),        # 6 NeoX segments (one wave per segment) / 12
+    (700, 32, 32, 128, 128),        # a token dealt to two waves: 2 x 4 NeoX segments / 2 x 8
+    (600, 64, 8, 128, 128),         # 3 x 3 / 2 x 9
+    (560, 28, 24, 128, 128),        # 7 as 4 + 3 (the last segment of the second wave is empty) / 2 x 7
+    (520, 40, 40, 128, 128),        # 2 x 5 / 2 x 10
 ])
 def test_rope_shapes_bit_exact(ops, dev, T, nq, nkv, D, R, is_neox):
     for packed in (False, True):

@@ -227,6 +227,25 @@ def test_fused_rope_append_one_wave_per_token(ops, dev, nq, nkv, is_neox, D, wri
     """Batches of 1024..4096 tokens take the kernel shape in which one wave covers a whole token
     (4097: one wave per segment again).  Checked bit for bit against the two stand-alone ops (each
     checked against its oracle elsewhere), with fewer appended rows than tokens."""
+    _fused_equals_rope_then_append(ops, dev, nq, nkv, is_neox, D, write_key, T)
+
+
+@pytest.mark.parametrize("T,nq,nkv,is_neox", [
+    (400, 32, 32, True),     # eight segments as two waves of four
+    (384, 64, 8, True),      # nine as three of three, the key heads in the last
+    (1000, 56, 8, True),     # eight as two of four; few key heads: dealt up to eight waves per unit
+    (420, 28, 24, True),     # seven as four and three: the second wave's last segment is empty
+    (400, 32, 32, False),    # interleaved pairs: sixteen segments as two waves of eight
+    (300, 40, 40, False),    # twenty as two of ten
+])
+@pytest.mark.parametrize("write_key", [False, True])
+def test_fused_rope_append_token_dealt_to_several_waves(ops, dev, T, nq, nkv, is_neox, write_key):
+    """Tokens of more segments than one wave takes, at batch sizes where they are dealt to two or
+    three waves of several segments each instead of one wave per segment."""
+    _fused_equals_rope_then_append(ops, dev, nq, nkv, is_neox, 128, write_key, T)
+
+
+def _fused_equals_rope_then_append(ops, dev, nq, nkv, is_neox, D, write_key, T):
     page_size, n = 16, T - 50
     g = gen(nq * 100 + nkv)
     pages = (n + page_size - 1) // page_size
