@@ -138,7 +138,8 @@ constexpr int kNtStore = 2;
 // constant), which leaves one resource and no per-segment selects in the kernel.  A token's
 // segment list is A's segments, then B's.
 //   geom  = head_bytes | embed_bytes << 16          (bytes of one head / of rot_dim/2)
-//   heads = heads of A | heads of B << 12 | slot_shift << 24 | (A is the key array) << 31
+//   heads = heads of A | heads of B << 12 | slot_shift << 24 | log2 gcd(chunks, 8) << 28 |
+//           (A is the key array) << 31     (the gcd field is filled in at launch)
 // slot_shift = log2(16-byte slots per head), at most 6; NeoX counts the slots of the x half,
 // GPT-J those of the whole rotated span.
 // Everything the first loads need sits in the first 56 bytes of the kernel arguments, which the
@@ -178,10 +179,18 @@ SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
   constexpr int SP = SPW == 1 ? kStreamStore : kNtStore;
   const uint32_t head_bytes = geom & 0xffffu, embed_bytes = geom >> 16;
   const uint32_t heads_a = heads & 0xfffu, heads_b = (heads >> 12) & 0xfffu;
-  const uint32_t sh = (heads >> 24) & 0x7fu;
+  const uint32_t sh = (heads >> 24) & 0x7u;
   const bool a_is_key = (heads & kRopeAIsKey) != 0;
   const int64_t tok = FLAT ? (int64_t)blockIdx.x : (int64_t)blockIdx.z * kMaxGridY + blockIdx.y;
-  const uint32_t chunk = FLAT ? 0u : blockIdx.x;
+  uint32_t chunk = FLAT ? 0u : blockIdx.x;
+  if constexpr (APPEND && !FLAT) {
+    // Workgroup ids go round the eight XCDs, and a token's key segments (twice the loads and
+    // stores of a query segment) sit at fixed places in its list: when the list length shares a
+    // factor g with 8 they would always land on the same 8 / g XCDs.  Exchanging chunks inside
+    // aligned groups of g, by an amount that steps every 8 / g tokens, spreads them over all eight.
+    const uint32_t lg = (heads >> 28) & 3u;  // log2 g, from the host
+    chunk ^= ((uint32_t)tok >> (3u - lg)) & ((1u << lg) - 1u);
+  }
   const uint32_t delta = (uint32_t)(delta0 + tok * delta_step);
   // A's row and, beyond it, B's: per-access validity is decided below (kClipped), the resource
   // only has to reach past B's row
@@ -365,8 +374,9 @@ struct RopeChunks {
 // 768 6.1 -> 5.7 (896: 7.0 against 7.2); 64 + 64 heads, 512 tokens 7.2 -> 6.4 (640 equal).  With
 // the append fused in the gain ends earlier, at five waves per unit (40 + 40 heads, 640 tokens
 // 8.9 -> 8.6, 768 10.4 against 10.5; 32 + 32 heads, 768 tokens 9.4 -> 8.1, 1024 equal), unless
-// the key heads are a small part of the token: 56 + 8 heads gain at every size measured (1024
-// tokens 10.1 -> 7.7 us, 1536 14.1 -> 12.0), 64 + 8 heads up to nine waves per unit.
+// the key heads are a small part of the token: 56 + 8 heads at 1024 tokens 10.0 -> 7.0 us and
+// still ahead at twelve waves per unit, 64 + 8 heads up to nine waves per unit (768 tokens
+// 7.2 -> 6.8, 896: 8.1 against 8.3).
 static RopeChunks plan_rope_chunks(int64_t segs, int64_t key_segs, int64_t tokens, int max_segs,
                                    bool append) {
   const int64_t units = compute_units();
@@ -374,8 +384,11 @@ static RopeChunks plan_rope_chunks(int64_t segs, int64_t key_segs, int64_t token
   p.chunks = (int)(segs < 1 ? 1 : segs);
   p.spw = 1;
   if (segs <= max_segs) {
-    const bool in_range = append ? tokens >= 4 * units && tokens <= 16 * units
-                                 : tokens >= 5 * units && 4 * tokens <= 41 * units;
+    // tokens of one or two segments (tensor-parallel shards: 8 + 1 heads): the whole token at
+    // every size measured, 3072 tokens 4.8 -> 4.5 us, 4608 6.3 -> 5.5, 8192 9.3 -> 8.4
+    const bool in_range = segs <= 2 ? tokens >= 5 * units
+                          : append  ? tokens >= 4 * units && tokens <= 16 * units
+                                    : tokens >= 5 * units && 4 * tokens <= 41 * units;
     if (in_range) {
       p.chunks = 1;
       p.spw = (int)(segs < 1 ? 1 : segs);
@@ -385,7 +398,7 @@ static RopeChunks plan_rope_chunks(int64_t segs, int64_t key_segs, int64_t token
   int64_t parts = (segs + max_segs - 1) / max_segs;
   if (segs % parts != 0 && segs % (parts + 1) == 0) ++parts;
   const int64_t waves = parts * tokens;
-  const int64_t lo = append ? 3 : 4, hi = append && 4 * key_segs > segs ? 5 : 8;
+  const int64_t lo = append ? 3 : 4, hi = !append ? 8 : 4 * key_segs > segs ? 5 : 9;
   if (waves >= lo * units && waves <= hi * units) {
     p.chunks = (int)parts;
     p.spw = (int)((segs + parts - 1) / parts);
@@ -466,7 +479,7 @@ static int launch_rope_piece(const RopeLaunch& l, int64_t segs, int64_t num_toke
                              const void* value, int64_t vsb, int write_key, const KvDest* d,
                              hipStream_t st) {
   if (segs <= 0) return SARATHI_OK;
-  const uint32_t sh = (l.heads >> 24) & 0x7fu;
+  const uint32_t sh = (l.heads >> 24) & 0x7u;
   const int64_t key_heads = (l.heads & kRopeAIsKey) ? (l.heads & 0xfffu) : ((l.heads >> 12) & 0xfffu);
   const RopeChunks plan =
       plan_rope_chunks(segs, ((key_heads << sh) + 63) >> 6, num_tokens,
@@ -494,6 +507,10 @@ static int launch_rope_piece(const RopeLaunch& l, int64_t segs, int64_t num_toke
     dr.nnz = d->nnz > t0 ? d->nnz - t0 : 0;
     value_r = reinterpret_cast<const char*>(value) + t0 * vsb;
   }
+  // see the chunk exchange in rope_wave()
+  uint32_t lg = 0;
+  while (lg < 3 && (plan.chunks & (1 << lg)) == 0) ++lg;
+  const uint32_t heads_arg = l.heads | (lg << 28);
   const dim3 block(64);
   const dim3 grid_full((unsigned)plan.chunks, kMaxGridY, (unsigned)full_z);
   const dim3 grid_rem = flat ? dim3((unsigned)rem) : dim3((unsigned)plan.chunks, (unsigned)rem, 1);
@@ -504,11 +521,12 @@ static int launch_rope_piece(const RopeLaunch& l, int64_t segs, int64_t num_toke
     if constexpr (APPEND)                                                                        \
       hipLaunchKernelGGL((rope_append_tok_kernel<DT, NEOX, SPW, FLAT, PAIRED>), GRID, block, 0,  \
                          st, L.positions, L.a, L.cache, L.a_stride_bytes, L.delta0,              \
-                         L.delta_step, L.geom, L.heads, VALUE, vsb, (uint32_t)write_key, DEST);  \
+                         L.delta_step, L.geom, heads_arg, VALUE, vsb, (uint32_t)write_key,       \
+                         DEST);                                                                  \
     else                                                                                         \
       hipLaunchKernelGGL((rope_tok_kernel<DT, NEOX, SPW, FLAT, PAIRED>), GRID, block, 0, st,     \
                          L.positions, L.a, L.cache, L.a_stride_bytes, L.delta0, L.delta_step,    \
-                         L.geom, L.heads);                                                       \
+                         L.geom, heads_arg);                                                     \
   } while (0)
 #define SK_ROPE_GO(SPW, FLAT, GRID, L, VALUE, DEST)                                              \
   do {                                                                                           \

@@ -349,7 +349,9 @@ def test_gelu_table_path_replayed_in_a_hip_graph(ops, dev):
 def _rope_case(ops, dev, dtype, T, nq, nkv, D, R, is_neox, packed, seed=1, prefill=None):
     g = gen(seed)
     cache = cos_sin_cache(8192, R, THETA_LLAMA3, dtype)
-    pos = hybrid_positions(T, prefill if prefill is not None else (T * 8) // 9, g)
+    # prefill positions start at 4096 and the table has 8192 rows
+    pos = hybrid_positions(T, prefill if prefill is not None else min((T * 8) // 9, 4096), g)
+    assert int(pos.max()) < cache.shape[0]
     if packed:
         qkv = randn((T, (nq + 2 * nkv) * D), g, dtype)
         want = qkv.clone()
@@ -404,6 +406,7 @@ def test_rope_llama3_8b_hybrid_batch_bit_exact(ops, dev, dtype, is_neox, packed)
     (600, 64, 8, 128, 128),         # 3 x 3 / 2 x 9
     (560, 28, 24, 128, 128),        # 7 as 4 + 3 (the last segment of the second wave is empty) / 2 x 7
     (520, 40, 40, 128, 128),        # 2 x 5 / 2 x 10
+    (5000, 8, 1, 128, 128),         # two segments: one wave per token at every batch size
 ])
 def test_rope_shapes_bit_exact(ops, dev, T, nq, nkv, D, R, is_neox):
     for packed in (False, True):

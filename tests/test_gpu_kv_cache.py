@@ -220,6 +220,7 @@ def test_fused_rope_append_equals_separate_ops(ops, dev, dtype, is_neox, nq, nkv
     (71, 1, True, 64),     # heads of 128 bytes (memory-order loads): Falcon-7B, five q segments + one
     (40, 8, True, 64),     # three segments, the key heads in the first half of theirs
     (9, 9, True, 64),      # ragged: nine heads in a segment of sixteen, for q and for k
+    (56, 8, True, 128),    # eight segments: per segment, chunks exchanged over all eight XCDs
 ])
 @pytest.mark.parametrize("write_key", [False, True])
 @pytest.mark.parametrize("T", [1700, 1024, 4096, 4097])
