@@ -19,6 +19,9 @@
 // a launch of N one-wave workgroups costs about 0.2 ns per workgroup in the
 // dispatcher alone, 3.5 us for the 11520 of the per-segment layout, and
 // multi-wave workgroups lose more to uneven compute-unit load than they gain.)
+// Tokens with more segments than that are dealt to two or three waves at mid-size batches
+// (plan_rope_chunks), and NeoX heads of 128 bytes are read in memory order with the x and y
+// vectors traded between lanes (trade_pairs).
 // The token's q row, k row and cos/sin cache row are scalar buffer resources
 // (the position is a scalar load issued first and consumed after the data loads
 // have been issued); lanes past the last head are clipped by the hardware range
