@@ -29,6 +29,9 @@ Sections (--section, comma separated, default all):
             beside the headline, not in it)
   cpu       `cpu_baseline`: the PyTorch CPU formulation of the same step on the host cores, and a
             CPU column for the per-op tables
+  models    (only when named; not part of "all") the four layer ops at the layer shapes of the model
+            families the reference serves, full width and tensor-parallel shards, at 1024, 2304 and
+            4608 tokens
 Per-op figures: `us` is the average over >= 100 back-to-back launches between two HIP events on
 the launch stream; `us_event_pair_median` is the median over the same number of launches with an
 event pair around every single call (it includes the events' own cost, about 1 us).  `roofline`
@@ -57,6 +60,7 @@ for _p in (ROOT, os.path.join(ROOT, "sarathi-serve_amd"), os.path.join(ROOT, "te
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = 2500.0
 SECTIONS = ("headline", "ceiling", "kv", "routing", "other", "moe", "cpu")
+EXTRA_SECTIONS = ("models",)   # run only when named
 
 T, H, NQ, NKV, D, DFF = 2304, 4096, 32, 8, 128, 14336
 PREFILL = 2048
@@ -156,9 +160,10 @@ def main():
         sys.exit("bench.py: this op library runs on one GPU; --gpus must be 1 "
                  "(the ops are per-token and never communicate)")
     want = set(SECTIONS) if args.section == "all" else set(args.section.split(","))
-    unknown = want - set(SECTIONS)
+    unknown = want - set(SECTIONS) - set(EXTRA_SECTIONS)
     if unknown:
-        sys.exit("bench.py: unknown section(s) %s; choose from %s" % (sorted(unknown), SECTIONS))
+        sys.exit("bench.py: unknown section(s) %s; choose from %s"
+                 % (sorted(unknown), SECTIONS + EXTRA_SECTIONS))
     if args.no_cpu_baseline:
         want.discard("cpu")
 
@@ -463,14 +468,15 @@ def main():
 
     # =========================================================================== other
     other_configs = None
-    if "other" in want:
+    if "other" in want or "models" in want:
         # C1: the fused norm at the 512-token shape that is also the CPU-sized case; C5: the four
         # ops at Llama-3-70B widths, T = 4608 (4096-token chunk + 512 decodes), one GPU, unsharded.
-        def measure_shape(Tn, Hn, nq, nkv, dff, which, prefill=None):
+        def measure_shape(Tn, Hn, nq, nkv, dff, which, prefill=None, head=D):
             rows = {}
             wn = dev_randn((Hn,))
             posn = hybrid_positions(Tn, prefill or Tn - Tn // 9, gen(4), prefill_start=4096,
                                     max_pos=8192).to(dev) if any("rotary" in w for w in which) else None
+            cache_n = cache_dev if head == D else cos_sin_cache(8192, head, THETA_LLAMA3, bf16).to(dev)
             plan = {
                 "fused_add_rms_norm": (4 * Tn * Hn * BF16 + Hn * BF16,
                                        lambda: (dev_randn((Tn, Hn)), dev_randn((Tn, Hn))),
@@ -478,11 +484,12 @@ def main():
                 "rms_norm": (2 * Tn * Hn * BF16 + Hn * BF16,
                              lambda: (dev_randn((Tn, Hn)), dev_randn((Tn, Hn))),
                              lambda a: LN.rms_norm(a[1], a[0], wn, 1e-5)),
-                "rotary_embedding": (2 * Tn * (nq + nkv) * D * BF16 + Tn * 8 + Tn * D * BF16,
-                                     lambda: dev_randn((Tn, (nq + 2 * nkv) * D)),
-                                     lambda a: ROPE.rotary_embedding(
-                                         posn, *a.split([nq * D, nkv * D, nkv * D], dim=-1)[:2], D,
-                                         cache_dev, True)),
+                "rotary_embedding": (2 * Tn * (nq + nkv) * head * BF16 + Tn * 8 + Tn * head * BF16,
+                                     # q and k views of a packed qkv buffer, cut outside the timed call
+                                     lambda: dev_randn((Tn, (nq + 2 * nkv) * head)).split(
+                                         [nq * head, nkv * head, nkv * head], dim=-1)[:2],
+                                     lambda a: ROPE.rotary_embedding(posn, a[0], a[1], head, cache_n,
+                                                                     True)),
                 "silu_and_mul": (3 * Tn * dff * BF16,
                                  lambda: (dev_randn((Tn, 2 * dff)),
                                           torch.empty((Tn, dff), dtype=bf16, device=dev)),
@@ -497,9 +504,9 @@ def main():
                               lambda a: ACT.gelu_fast(a[1], a[0])),
                 "rotary_embedding (GPT-J layout)": (
                     2 * Tn * (nq + nkv) * D * BF16 + Tn * 8 + Tn * D * BF16,
-                    lambda: dev_randn((Tn, (nq + 2 * nkv) * D)),
-                    lambda a: ROPE.rotary_embedding(
-                        posn, *a.split([nq * D, nkv * D, nkv * D], dim=-1)[:2], D, cache_dev, False)),
+                    lambda: dev_randn((Tn, (nq + 2 * nkv) * D)).split([nq * D, nkv * D, nkv * D],
+                                                                      dim=-1)[:2],
+                    lambda a: ROPE.rotary_embedding(posn, a[0], a[1], D, cache_dev, False)),
             }
             for name in which:
                 nbytes, make, fn = plan[name]
@@ -512,6 +519,7 @@ def main():
                 torch.cuda.empty_cache()
             return rows
 
+    if "other" in want:
         other_configs = {
             "rest of the module surface at the Llama-3-8B batch, T=2304: gelu_new / gelu_fast "
             "[2304, 14336], rotary_embedding with interleaved (GPT-J) pairs":
@@ -531,6 +539,34 @@ def main():
                               ["fused_add_rms_norm", "rms_norm", "rotary_embedding", "silu_and_mul"]),
         }
         out["other_configs"] = other_configs
+
+    # =========================================================================== models
+    if "models" in want:
+        # Layer shapes of the model families the reference serves (sarathi/model_executor/models/):
+        # hidden, query + key heads of head_size, intermediate size (0: no gated activation); "tp N"
+        # is one GPU's share under the reference's tensor parallelism, whose norms see the full
+        # hidden size.  A 2048-token chunk (or all but a ninth of the batch) plus decodes.
+        shapes = [
+            ("Llama-3-8B / Mistral-7B / Mixtral-8x7B", 4096, 32, 8, 128, 14336),
+            ("Llama-2-7B", 4096, 32, 32, 128, 11008),
+            ("Llama-2-13B / InternLM-20B", 5120, 40, 40, 128, 13824),
+            ("Yi-34B", 7168, 56, 8, 128, 20480),
+            ("Llama-3-70B", 8192, 64, 8, 128, 28672),
+            ("Qwen-72B", 8192, 64, 64, 128, 24576),
+            ("Falcon-7B", 4544, 71, 1, 64, 0),
+            ("Falcon-40B", 8192, 128, 8, 64, 0),
+            ("Llama-3-70B tp 4", 8192, 16, 2, 128, 7168),
+            ("Llama-3-70B tp 8", 8192, 8, 1, 128, 3584),
+        ]
+        models = {}
+        for name, Hn, nq, nkv, head, dff in shapes:
+            which = ["rms_norm", "fused_add_rms_norm", "rotary_embedding"] + (["silu_and_mul"] if dff else [])
+            models[name] = {
+                "hidden": Hn, "heads": [nq, nkv], "head_size": head, "intermediate": dff,
+                "tokens": {str(Tn): measure_shape(Tn, Hn, nq, nkv, dff, which,
+                                                  prefill=min(2048, Tn - Tn // 9), head=head)
+                           for Tn in (1024, 2304, 4608)}}
+        out["model_shapes"] = models
 
     # =========================================================================== moe
     if "moe" in want:
