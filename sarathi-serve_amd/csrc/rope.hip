@@ -139,7 +139,7 @@ constexpr int kNtStore = 2;
 // starts lower in memory, and B is reached THROUGH A's per-token buffer resource at byte offset
 // delta0 + token * delta_step (callers pass views of one packed qkv buffer, so this is a small
 // constant), which leaves one resource and no per-segment selects in the kernel.  A token's
-// segment list is A's segments, then B's.
+// list of heads is A's heads, then B's, cut into segments of 64 slots.
 //   geom  = head_bytes | embed_bytes << 16          (bytes of one head / of rot_dim/2)
 //   heads = heads of A | heads of B << 12 | slot_shift << 24 | log2 gcd(chunks, 8) << 28 |
 //           (A is the key array) << 31     (the gcd field is filled in at launch)
@@ -198,7 +198,10 @@ SK_DEV void rope_wave(const int64_t* __restrict__ positions, void* a,
   // A's row and, beyond it, B's: per-access validity is decided below (kClipped), the resource
   // only has to reach past B's row
   const rsrc_t r = make_rsrc(reinterpret_cast<char*>(a) + tok * a_stride_bytes, 0x7fffffffu);
-  const uint32_t a_pad = (((heads_a << sh) + 63u) >> 6) << (6 - sh);  // A's heads in whole segments
+  // B's heads follow A's in the token's list.  With the append fused in, A's span is padded to
+  // whole segments, so that a segment is all key heads or none (the append decisions are then
+  // uniform over the wave); without it B's first head takes the lane after A's last.
+  const uint32_t a_pad = APPEND ? (((heads_a << sh) + 63u) >> 6) << (6 - sh) : heads_a;
   const uint32_t slot = threadIdx.x & ((1u << sh) - 1u);
   // PAIRED (sh == 2): the lane's piece of its head in memory order, see trade_pairs()
   const uint32_t h0 = chunk * (uint32_t)(SPW << (6 - sh)) + (threadIdx.x >> (PAIRED ? 3 : sh));
@@ -417,7 +420,7 @@ struct RopeAnchor {
   int64_t segs[2];
 };
 static RopeAnchor plan_rope_anchor(const RopeArgs& a, int eb, int slots, int slot_shift,
-                                   uint32_t geom) {
+                                   uint32_t geom, bool append) {
   const int64_t qsb = a.q_stride * eb, ksb = a.k_stride * eb;
   const int64_t q_row = (int64_t)a.num_heads * a.head_size * eb;
   const int64_t k_row = (int64_t)a.num_kv_heads * a.head_size * eb;
@@ -427,6 +430,9 @@ static RopeAnchor plan_rope_anchor(const RopeArgs& a, int eb, int slots, int slo
   const int64_t d_first = k - q, d_last = d_first + last * (ksb - qsb);  // key row - query row
   const int64_t q_blocks = ((int64_t)a.num_heads * slots + 63) / 64;
   const int64_t k_blocks = ((int64_t)a.num_kv_heads * slots + 63) / 64;
+  // segments of a token whose two rows go out in one launch: see a_pad in rope_wave()
+  const int64_t joined =
+      append ? q_blocks + k_blocks : ((int64_t)(a.num_heads + a.num_kv_heads) * slots + 63) / 64;
   const int64_t reach = (int64_t)kClipped - 64;  // offsets, + embed_bytes, must stay below kClipped
   const uint32_t sh = (uint32_t)slot_shift << 24;
   RopeAnchor p;
@@ -435,12 +441,12 @@ static RopeAnchor plan_rope_anchor(const RopeArgs& a, int eb, int slots, int slo
     p.pieces = 1;  // A = query, B = key
     p.l[0] = {a.positions, q, a.cache, qsb, d_first, ksb - qsb, geom,
               (uint32_t)a.num_heads | ((uint32_t)a.num_kv_heads << 12) | sh};
-    p.segs[0] = q_blocks + k_blocks;
+    p.segs[0] = joined;
   } else if (d_first <= 0 && d_last <= 0 && -d_first + q_row < reach && -d_last + q_row < reach) {
     p.pieces = 1;  // A = key, B = query
     p.l[0] = {a.positions, k, a.cache, ksb, -d_first, qsb - ksb, geom,
               (uint32_t)a.num_kv_heads | ((uint32_t)a.num_heads << 12) | sh | kRopeAIsKey};
-    p.segs[0] = q_blocks + k_blocks;
+    p.segs[0] = joined;
   } else {
     p.pieces = 2;  // too far apart (or crossing): each array on its own
     p.l[0] = {a.positions, q, a.cache, qsb, 0, 0, geom, (uint32_t)a.num_heads | sh};
@@ -605,7 +611,7 @@ static int launch_rope(const RopeArgs& a, hipStream_t st) {
     return launch_status();
   }
   const uint32_t geom = (uint32_t)head_bytes | ((uint32_t)(embed * EB) << 16);
-  const RopeAnchor plan = plan_rope_anchor(a, EB, slots, slot_shift, geom);
+  const RopeAnchor plan = plan_rope_anchor(a, EB, slots, slot_shift, geom, false);
   for (int i = 0; i < plan.pieces; ++i) {
     const int rc = launch_rope_piece<DT, NEOX, false>(plan.l[i], plan.segs[i], a.num_tokens,
                                                       nullptr, 0, 0, nullptr, st);
@@ -694,7 +700,7 @@ static int launch_rope_append(const RopeArgs& a, const void* value, int64_t v_st
     return launch_status();
   }
   const uint32_t geom = (uint32_t)head_bytes | ((uint32_t)(embed * EB) << 16);
-  const RopeAnchor plan = plan_rope_anchor(a, EB, slots, slot_shift, geom);
+  const RopeAnchor plan = plan_rope_anchor(a, EB, slots, slot_shift, geom, true);
   for (int i = 0; i < plan.pieces; ++i) {
     const int rc = launch_rope_piece<DT, NEOX, true>(plan.l[i], plan.segs[i], a.num_tokens, value,
                                                      vsb, write_key, &d, st);
