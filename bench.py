@@ -175,6 +175,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     LN, ACT, ROPE, MOE = ops.layernorm_ops, ops.activation_ops, ops.pos_encoding_ops, ops.moe_ops
+    KV = ops.kv_cache_ops
     bf16 = torch.bfloat16
     torch.manual_seed(1)
     reps = max(args.steps, MIN_REPS)
@@ -379,7 +380,6 @@ def main():
     if "kv" in want:
         # paged KV cache of the hybrid batch: one prompt chunk continuing a 4096-token request and
         # 256 decode requests with contexts of 1..3000 tokens, pages handed out in random order
-        from sarathi_amd import kv_cache_ops as KV
         from sarathi_amd import layers as LAYERS
         import numpy as np
         rng = np.random.default_rng(5)
@@ -477,6 +477,19 @@ def main():
             posn = hybrid_positions(Tn, prefill or Tn - Tn // 9, gen(4), prefill_start=4096,
                                     max_pos=8192).to(dev) if any("rotary" in w for w in which) else None
             cache_n = cache_dev if head == D else cos_sin_cache(8192, head, THETA_LLAMA3, bf16).to(dev)
+            if "rotary_embedding + KV append" in which:
+                # one request that appends all Tn tokens to pages of 16 entries in shuffled order
+                n_pages = (Tn + 15) // 16
+                ap_b = torch.zeros(Tn, dtype=torch.int32, device=dev)
+                ap_pos = torch.arange(Tn, dtype=torch.int32, device=dev)
+                ap_pages = torch.randperm(n_pages, generator=gen(7)).to(torch.int32).to(dev)
+                ap_indptr = torch.tensor([0, n_pages], dtype=torch.int32, device=dev)
+
+                def mk_append():
+                    q, k, v = dev_randn((Tn, (nq + 2 * nkv) * head)).split(
+                        [nq * head, nkv * head, nkv * head], dim=-1)
+                    cache = torch.empty((n_pages, 2, 16, nkv, head), dtype=bf16, device=dev)
+                    return (q, k, v, (cache[:, 0], cache[:, 1]))
             plan = {
                 "fused_add_rms_norm": (4 * Tn * Hn * BF16 + Hn * BF16,
                                        lambda: (dev_randn((Tn, Hn)), dev_randn((Tn, Hn))),
@@ -490,6 +503,12 @@ def main():
                                          [nq * head, nkv * head, nkv * head], dim=-1)[:2],
                                      lambda a: ROPE.rotary_embedding(posn, a[0], a[1], head, cache_n,
                                                                      True)),
+                "rotary_embedding + KV append": (
+                    (2 * Tn * nq + 4 * Tn * nkv) * head * BF16 + 24 * Tn + Tn * head * BF16,
+                    lambda: mk_append(),
+                    lambda a: KV.rotary_embedding_append_paged_kv(
+                        posn, a[0], a[1], a[2], head, cache_n, True, ap_b, ap_pos, a[3], ap_pages,
+                        ap_indptr)),
                 "silu_and_mul": (3 * Tn * dff * BF16,
                                  lambda: (dev_randn((Tn, 2 * dff)),
                                           torch.empty((Tn, dff), dtype=bf16, device=dev)),
@@ -560,7 +579,8 @@ def main():
         ]
         models = {}
         for name, Hn, nq, nkv, head, dff in shapes:
-            which = ["rms_norm", "fused_add_rms_norm", "rotary_embedding"] + (["silu_and_mul"] if dff else [])
+            which = (["rms_norm", "fused_add_rms_norm", "rotary_embedding", "rotary_embedding + KV append"]
+                     + (["silu_and_mul"] if dff else []))
             models[name] = {
                 "hidden": Hn, "heads": [nq, nkv], "head_size": head, "intermediate": dff,
                 "tokens": {str(Tn): measure_shape(Tn, Hn, nq, nkv, dff, which,
