@@ -20,10 +20,11 @@ namespace sarathi_hip {
 #define SARATHI_KV_STORE_POLICY 0
 #endif
 constexpr int kKvStore = SARATHI_KV_STORE_POLICY;
-// The same for the rotary embedding fused with the append: there the cache stores leave the wave
-// together with eight in-place query stores per lane, and a non-temporal hint (2) keeps them from
-// displacing the rows other waves are still reading (2304 tokens: 10.5 -> 9.7 us; the stand-alone
-// append is fastest with the default policy, 4.2 against 4.4 us).
+// The same for the rotary embedding fused with the append, in the waves that take several
+// segments of a token: there the cache stores leave the wave together with eight in-place query
+// stores per lane, and a non-temporal hint (2) keeps them from displacing the rows other waves are
+// still reading (2304 tokens: 10.5 -> 9.7 us; the stand-alone append and the fused kernel's
+// one-segment waves are fastest with the default policy).
 #ifndef SARATHI_KV_STORE_POLICY_FUSED
 #define SARATHI_KV_STORE_POLICY_FUSED 2
 #endif
