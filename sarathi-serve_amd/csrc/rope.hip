@@ -384,9 +384,10 @@ struct RopeChunks {
 // 768 6.1 -> 5.7 (896: 7.0 against 7.2); 64 + 64 heads, 512 tokens 7.2 -> 6.4 (640 equal).  With
 // the append fused in the gain ends earlier, at five waves per unit (40 + 40 heads, 640 tokens
 // 8.9 -> 8.6, 768 10.4 against 10.5; 32 + 32 heads, 768 tokens 9.4 -> 8.1, 1024 equal), unless
-// the key heads are a small part of the token: 56 + 8 heads at 1024 tokens 10.0 -> 7.0 us and
-// still ahead at twelve waves per unit, 64 + 8 heads up to nine waves per unit (768 tokens
-// 7.2 -> 6.8, 896: 8.1 against 8.3).
+// the key heads are a small part of the token, where it lasts to twelve waves per unit: 56 + 8
+// heads at 1024 tokens 9.4 -> 6.8 us, 1536 12.5 -> 11.2 (2304 equal, behind from there); 64 + 8
+// heads at 1024 tokens 8.8 -> 7.5 (1280 equal); 40 + 8 heads at 1280 tokens 8.3 -> 6.8, 1536
+// 9.4 -> 8.8 (2048 behind).
 static RopeChunks plan_rope_chunks(int64_t segs, int64_t key_segs, int64_t tokens, int max_segs,
                                    bool append) {
   const int64_t units = compute_units();
@@ -408,7 +409,7 @@ static RopeChunks plan_rope_chunks(int64_t segs, int64_t key_segs, int64_t token
   int64_t parts = (segs + max_segs - 1) / max_segs;
   if (segs % parts != 0 && segs % (parts + 1) == 0) ++parts;
   const int64_t waves = parts * tokens;
-  const int64_t lo = append ? 3 : 4, hi = !append ? 8 : 4 * key_segs > segs ? 5 : 9;
+  const int64_t lo = append ? 3 : 4, hi = !append ? 8 : 4 * key_segs > segs ? 5 : 12;
   if (waves >= lo * units && waves <= hi * units) {
     p.chunks = (int)parts;
     p.spw = (int)((segs + parts - 1) / parts);
