@@ -7,7 +7,8 @@ counts, widths, dtypes and token counts around every multiple of the compute-uni
 rule could use, so that a rule added later is exercised on both sides without a test of its own.
 Each case goes through the op namespace -> C ABI and is compared with the oracle (rotary: bit for
 bit; norms: the dtype tolerance of the dense-op tests) or, for the fused append, bit for bit with
-the two stand-alone ops.
+the two stand-alone ops.  The activations, whose only rule is whole vectors or not, get a smaller
+sweep over widths, strides and dtypes.
 """
 import random
 
@@ -172,3 +173,42 @@ def test_rms_norm_and_fused_sweep_match_oracle(ops, dev, case):
     assert torch.equal(gr.cpu(), wr), "residual = T(x + r) must be bit-exact"
     assert_close_dtype(gx, wx, **tol)
     assert bool((gx_buf[:, H:] == 0).all()) and bool((gr_buf[:, H:] == 0).all())
+
+
+ACT_CASES = 30
+
+
+@pytest.mark.parametrize("case", range(ACT_CASES))
+def test_activation_sweep_matches_oracle(ops, dev, case):
+    """silu_and_mul (row views with strides of their own) and gelu_new / gelu_fast over widths that
+    are and are not whole 16-byte vectors or whole 1 KiB segments."""
+    rng = random.Random(6000 + case)
+    dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
+    per_vec = 4 if dtype == torch.float32 else 8
+    d = rng.choice([1, 3, per_vec, 5 * per_vec, 64 * per_vec, 64 * per_vec + per_vec, 1000, 3584,
+                    4095, 11008, 14336])
+    T = rng.choice([1, 2, 37, 300, 1025, 2304]) if d > 4096 else _token_counts(rng, 1, top=3000)[0]
+    g = gen(7000 + case)
+    if dtype == torch.float32:
+        tol = dict(atol=2e-6, rtol=2e-5, max_ulps=None, max_mismatch_frac=1.0)
+    else:
+        tol = dict(atol=1e-2, rtol=1e-2, max_ulps=2, max_mismatch_frac=5e-3)
+    x = randn((T, 2 * d), g, dtype, std=2.0)
+    want = torch.empty((T, d), dtype=dtype)
+    c_oracle.silu_and_mul(want, x)
+    pad = per_vec * rng.choice([0, 0, 2])
+    in_buf = torch.zeros((T, 2 * d + pad), dtype=dtype, device=dev)
+    out_buf = torch.zeros((T, d + 2 * pad), dtype=dtype, device=dev)
+    in_buf[:, :2 * d].copy_(x)
+    ops.activation_ops.silu_and_mul(out_buf[:, :d], in_buf[:, :2 * d])
+    assert_close_dtype(out_buf[:, :d], want, **tol)
+    assert bool((out_buf[:, d:] == 0).all())
+
+    name = rng.choice(["gelu_new", "gelu_fast"])
+    xg = x[:, :d].contiguous()
+    wantg = torch.empty_like(xg)
+    getattr(c_oracle, name)(wantg, xg)
+    gotg = torch.empty_like(xg, device=dev)
+    getattr(ops.activation_ops, name)(gotg, xg.to(dev))
+    tol["max_mismatch_frac"] = max(tol["max_mismatch_frac"], 2e-2)
+    assert_close_dtype(gotg, wantg, **tol)
