@@ -9,10 +9,10 @@
 //          them in registers and writes both vectors back;
 //   GPT-J: x and y interleave, so one 16-byte vector already holds whole
 //          pairs; cos and sin come from two half-width loads.
-// 64 consecutive slots of a token's q row or of its k row (8 heads of 128 at
-// bf16) form a segment.  A workgroup is ONE wave that takes up to five NeoX
-// (ten GPT-J) consecutive segments of one token's list (q segments, then k
-// segments): at Llama-3-8B's 32 + 8 heads that is the whole token, so its position and its
+// 64 consecutive slots of a token's list of heads (the q heads, then the k heads;
+// 8 heads of 128 at bf16) form a segment.  A workgroup is ONE wave that takes up
+// to five NeoX (ten GPT-J) consecutive segments of one token:
+// at Llama-3-8B's 32 + 8 heads that is the whole token, so its position and its
 // cos/sin row are fetched once, all of its loads are in flight before the first
 // result is needed, and the launch has one workgroup per token.  (Measured on
 // MI355X at 2304 tokens: one wave per segment 9.3 us, one wave per token 8.1 us;
