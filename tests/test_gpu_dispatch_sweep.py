@@ -10,6 +10,7 @@ bit; norms: the dtype tolerance of the dense-op tests) or, for the fused append,
 the two stand-alone ops.  The activations, whose only rule is whole vectors or not, get a smaller
 sweep over widths, strides and dtypes.
 """
+import os
 import random
 
 import pytest
@@ -19,6 +20,11 @@ from helpers import THETA_LLAMA3, assert_close_dtype, cos_sin_cache, gen, hybrid
 from oracle import c_oracle
 
 pytestmark = pytest.mark.gpu
+
+# A longer sweep on request: SARATHI_SWEEP_SCALE multiplies the number of cases of every sweep,
+# SARATHI_SWEEP_OFFSET shifts all seeds.
+_SCALE = int(os.environ.get("SARATHI_SWEEP_SCALE", "1"))
+_OFFSET = int(os.environ.get("SARATHI_SWEEP_OFFSET", "0"))
 
 
 def _units():
@@ -50,12 +56,12 @@ def _rope_bits_equal(got, want):
     assert torch.equal(got.view(torch.int16)[nz], want.view(torch.int16)[nz])
 
 
-ROPE_CASES = 48
+ROPE_CASES = 48 * _SCALE
 
 
 @pytest.mark.parametrize("case", range(ROPE_CASES))
 def test_rotary_embedding_sweep_bit_exact(ops, dev, case):
-    rng = random.Random(1000 + case)
+    rng = random.Random(1000 + case + _OFFSET)
     nq = rng.choice([1, 3, 8, 9, 16, 20, 24, 28, 32, 40, 48, 56, 64, 71])
     nkv = rng.choice([1, 2, 4, 8, nq]) if rng.random() < 0.8 else rng.randint(1, nq)
     nkv = min(nkv, nq)
@@ -86,12 +92,12 @@ def test_rotary_embedding_sweep_bit_exact(ops, dev, case):
         _rope_bits_equal(gk.cpu(), wk)
 
 
-APPEND_CASES = 32
+APPEND_CASES = 32 * _SCALE
 
 
 @pytest.mark.parametrize("case", range(APPEND_CASES))
 def test_fused_rope_append_sweep_equals_separate_ops(ops, dev, case):
-    rng = random.Random(2000 + case)
+    rng = random.Random(2000 + case + _OFFSET)
     nq = rng.choice([8, 9, 16, 24, 28, 32, 40, 48, 56, 64, 71])
     nkv = min(nq, rng.choice([1, 2, 4, 8, 8, nq]))
     D = rng.choice([128, 128, 64])
@@ -129,12 +135,12 @@ def test_fused_rope_append_sweep_equals_separate_ops(ops, dev, case):
         assert torch.equal(k[:n], qkv.split([nq * D, nkv * D, nkv * D], dim=-1)[1][:n])
 
 
-NORM_CASES = 48
+NORM_CASES = 48 * _SCALE
 
 
 @pytest.mark.parametrize("case", range(NORM_CASES))
 def test_rms_norm_and_fused_sweep_match_oracle(ops, dev, case):
-    rng = random.Random(4000 + case)
+    rng = random.Random(4000 + case + _OFFSET)
     dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
     per_vec = 4 if dtype == torch.float32 else 8
     if rng.random() < 0.7:     # whole vectors: widths around every vector count a rule may use
@@ -175,14 +181,14 @@ def test_rms_norm_and_fused_sweep_match_oracle(ops, dev, case):
     assert bool((gx_buf[:, H:] == 0).all()) and bool((gr_buf[:, H:] == 0).all())
 
 
-ACT_CASES = 30
+ACT_CASES = 30 * _SCALE
 
 
 @pytest.mark.parametrize("case", range(ACT_CASES))
 def test_activation_sweep_matches_oracle(ops, dev, case):
     """silu_and_mul (row views with strides of their own) and gelu_new / gelu_fast over widths that
     are and are not whole 16-byte vectors or whole 1 KiB segments."""
-    rng = random.Random(6000 + case)
+    rng = random.Random(6000 + case + _OFFSET)
     dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
     per_vec = 4 if dtype == torch.float32 else 8
     d = rng.choice([1, 3, per_vec, 5 * per_vec, 64 * per_vec, 64 * per_vec + per_vec, 1000, 3584,
