@@ -153,6 +153,11 @@ def main():
                     help="moe section: spread every expert's slots evenly over its slot blocks before "
                          "the GEMMs (layers.balance_blocks) or leave moe_align_block_size's greedy fill "
                          "(the library's default)")
+    ap.add_argument("--moe-riders", choices=["on", "off"], default="on",
+                    help="moe section, row-major weights at 256-slot blocks: the slots of an expert's "
+                         "partly filled last block ride with the workgroups of its full blocks "
+                         "(moe_ops.moe_plan_riders; the library's default) or get workgroups of "
+                         "their own")
     ap.add_argument("--moe-block-m", type=int, default=0,
                     help="moe section: slot-block size of the grouped GEMMs (0 = the library's choice)")
     args = ap.parse_args()
@@ -597,6 +602,7 @@ def main():
         import importlib
         from sarathi_amd import layers
         importlib.import_module("sarathi_amd.layers.fused_moe").BALANCE_BLOCKS = args.moe_balance == "on"
+        importlib.import_module("sarathi_amd.layers.fused_moe").RIDERS = args.moe_riders == "on"
         E, k, Hm, I = 8, 2, 4096, 14336
 
         def timeit_ms(fn, n=20):
@@ -630,7 +636,7 @@ def main():
             w1.fill_(0.0078125)
             w2.fill_(0.0078125)
         forward = {}
-        for Tn in (16, 1024, 4096):
+        for Tn in (16, 1024, 2048, 4096):
             x = torch.randn((Tn, Hm), device=dev, dtype=torch.float32).to(bf16)
             if args.moe_data == "constant":
                 x.fill_(0.0078125)
@@ -667,14 +673,18 @@ def main():
                 torch.cuda.empty_cache()
             else:
                 b1, b2, pk, wa, wb = w1, w2, False, w1, w2
+            rd = None
+            if args.moe_riders == "on" and label == "row_major" and bm == 256 and args.moe_balance != "on":
+                rd = torch.empty((e_ids.numel(),), dtype=torch.int32, device=dev)
+                MOE.moe_plan_riders(s_ids, e_ids, p_pad, Tn * k, bm, rd)
             ms1 = timeit_ms(lambda: MOE.moe_grouped_gemm(
-                x, b1, c1, tw_m, s_ids, e_ids, p_pad, Tn * k, bm, k, False, pk, 2 * I))
+                x, b1, c1, tw_m, s_ids, e_ids, p_pad, Tn * k, bm, k, False, pk, 2 * I, False, rd))
             ms_act = timeit_ms(lambda: ACT.silu_and_mul(c2, c1.view(-1, 2 * I)))
             ms1s = timeit_ms(lambda: MOE.moe_grouped_gemm(
-                x, b1, c2, tw_m, s_ids, e_ids, p_pad, Tn * k, bm, k, False, pk, 2 * I, True))
+                x, b1, c2, tw_m, s_ids, e_ids, p_pad, Tn * k, bm, k, False, pk, 2 * I, True, rd))
             ACT.silu_and_mul(c2, c1.view(-1, 2 * I))
             ms2 = timeit_ms(lambda: MOE.moe_grouped_gemm(
-                c2, b2, c3, tw_m, s_ids, e_ids, p_pad, Tn * k, bm, 1, True, pk, Hm))
+                c2, b2, c3, tw_m, s_ids, e_ids, p_pad, Tn * k, bm, 1, True, pk, Hm, False, rd))
             ms_all = timeit_ms(lambda: layers.fused_moe(x, wa, wb, logits, k, True,
                                                         override_config=config))
             gemms[label] = {
@@ -688,7 +698,8 @@ def main():
                      "bf16, %s data, %s routing, slot blocks %s, back-to-back launches (weights "
                      "warm in L2/MALL as far as they fit)"
                      % (args.moe_data, args.moe_routing,
-                        "filled evenly per expert" if args.moe_balance == "on" else "filled greedily"),
+                        "filled evenly per expert" if args.moe_balance == "on"
+                        else "filled greedily, riders" if args.moe_riders == "on" else "filled greedily"),
             "peak": "2500 TFLOP/s dense bf16 MFMA; 8 TB/s HBM",
             "fused_moe_forward_row_major": forward, "at_4096_tokens": gemms}
 

@@ -376,6 +376,32 @@ int sarathi_moe_balance_blocks(const int32_t* sorted_in, int32_t* sorted_out,
                                int granule, int rows_per_block, void* stream);
 
 /*
+ * No counterpart in the reference: riders for the grouped GEMM.  moe_align_block_size fills an
+ * expert's blocks greedily (fused_moe.py:151-204), so an expert's last block is often nearly
+ * empty, and a workgroup of the GEMM that works on such a block still pulls the expert's whole
+ * weight tile through its compute unit.  sarathi_moe_plan_riders looks at moe_align_block_size's
+ * outputs for block_m = 256 and writes one int32 per slot block into `riders`: the first slot of
+ * a 32-slot tile of the same expert's last block that this block's workgroups multiply as well,
+ * -1 for none, -2 for a last block all of whose tiles ride with others (the GEMM skips it).  A
+ * last block rides when it holds at most as many 32-slot tiles as the expert has full blocks.
+ * sarathi_moe_grouped_gemm_riders is sarathi_moe_grouped_gemm with that table: row-major weights,
+ * block_m = 256, bfloat16 / float16 (anything else: SARATHI_ERR_UNSUPPORTED); same results bit
+ * for bit (a slot's dot products do not depend on which workgroup forms them).  The sorted ids
+ * must be in moe_align_block_size's greedy order (not rewritten by sarathi_moe_balance_blocks).
+ */
+int sarathi_moe_plan_riders(const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                            const int32_t* num_tokens_post_padded, int64_t num_valid_tokens,
+                            int64_t sorted_len, int block_m, int32_t* riders, int64_t riders_len,
+                            void* stream);
+int sarathi_moe_grouped_gemm_riders(const void* a, const void* b, void* c, const float* topk_weights,
+                                    const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                    const int32_t* num_tokens_post_padded, int64_t num_valid_tokens,
+                                    int64_t sorted_len, int64_t n, int64_t k, int64_t a_row_stride,
+                                    int64_t b_expert_stride, int64_t c_row_stride, int block_m,
+                                    int top_k, int epilogue, int b_layout, int dtype,
+                                    const int32_t* riders, void* stream);
+
+/*
  * No counterpart in the reference: how many equal ranges of a slot block the waves of the
  * sarathi_moe_grouped_gemm kernel for (block_m, b_layout) split between them (1 or 2; each range
  * is swept by its own waves, 32 slots at a time, and ranges without a valid slot in a tile are

@@ -23,7 +23,8 @@ OBJ_DIR = os.path.join(HERE, "build", "obj")
 
 HIP_SOURCES = ["rms_norm.hip", "gated_act.hip", "rope.hip", "moe_topk.hip", "moe_align.hip",
                "moe_gemm.hip", "moe_gemm_wide.hip", "moe_sum.hip", "kv_cache.hip",
-               "moe_fused_routing.hip", "stream_copy.hip", "moe_balance.hip", "moe_gemm_f32.hip"]
+               "moe_fused_routing.hip", "stream_copy.hip", "moe_balance.hip", "moe_gemm_f32.hip",
+               "moe_gemm_rider.hip"]
 CXX_SOURCES = ["abi_misc.cpp"]
 
 ABI_LIB = os.path.join(LIB_DIR, "libsarathi_ops_hip.so")

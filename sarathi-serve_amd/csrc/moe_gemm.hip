@@ -305,6 +305,9 @@ static int launch_moe_gemm(const MoeGemmArgs& g, int epilogue, bool packed, hipS
 // moe_gemm_wide.hip: row-major weights at 64-, 128- and 256-slot blocks, four waves
 int launch_moe_gemm_wide(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, int dtype,
                          hipStream_t st);
+// moe_gemm_rider.hip: row-major weights at 256-slot blocks, with riders
+int launch_moe_gemm_rider(MoeGemmArgs g, int64_t out_cols, int epilogue, int dtype,
+                         const int32_t* ride, hipStream_t st);
 // moe_gemm_f32.hip: float32 tensors
 int launch_moe_gemm_f32(const void* a, const void* b, void* c, const float* topk_weights,
                         const int32_t* sorted_token_ids, const int32_t* expert_ids,
@@ -326,17 +329,13 @@ extern "C" int sarathi_moe_gemm_slot_rows(int block_m, int b_layout) {
   return block_m == 256 ? 2 : 1;
 }
 
-extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
-                                        const float* topk_weights,
-                                        const int32_t* sorted_token_ids,
-                                        const int32_t* expert_ids,
-                                        const int32_t* num_tokens_post_padded,
-                                        int64_t num_valid_tokens, int64_t sorted_len, int64_t n,
-                                        int64_t k, int64_t a_row_stride, int64_t b_expert_stride,
-                                        int64_t c_row_stride, int block_m, int top_k,
-                                        int epilogue, int b_layout, int dtype,
-                                        void* stream) {
-  using namespace sarathi_hip;
+namespace sarathi_hip {
+static int grouped_gemm(const void* a, const void* b, void* c, const float* topk_weights,
+                        const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                        const int32_t* num_tokens_post_padded, int64_t num_valid_tokens,
+                        int64_t sorted_len, int64_t n, int64_t k, int64_t a_row_stride,
+                        int64_t b_expert_stride, int64_t c_row_stride, int block_m, int top_k,
+                        int epilogue, int b_layout, int dtype, const int32_t* ride, void* stream) {
   if (!a || !b || !c || !sorted_token_ids || !expert_ids || !num_tokens_post_padded)
     return SARATHI_ERR_INVALID_ARG;
   if (epilogue != SARATHI_MOE_EPILOGUE_NONE && epilogue != SARATHI_MOE_EPILOGUE_ROUTED_WEIGHT &&
@@ -353,6 +352,9 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
     return SARATHI_ERR_INVALID_ARG;
   const bool packed = b_layout == SARATHI_MOE_B_PACKED;
   if (packed && b_expert_stride < (n + 31) / 32 * 32 * k) return SARATHI_ERR_INVALID_ARG;
+  // riders exist in one kernel only: row-major 16-bit weights at 256-slot blocks
+  if (ride && (packed || block_m != 256 || (dtype != kBF16 && dtype != kF16)))
+    return SARATHI_ERR_UNSUPPORTED;
   if (dtype == kF32)
     return launch_moe_gemm_f32(a, b, c, topk_weights, sorted_token_ids, expert_ids,
                                num_tokens_post_padded, num_valid_tokens, sorted_len, n, k,
@@ -396,6 +398,7 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
   const int mw = epilogue;
   // row-major weights run the four-wave kernel of moe_gemm_wide.hip from 64-slot blocks on (32-slot
   // wave tiles for decode-size batches, 128 x 128 wave tiles at 256-slot blocks)
+  if (ride) return launch_moe_gemm_rider(g, c_cols, mw, dtype, ride, st);
   if (!packed && block_m >= 64) return launch_moe_gemm_wide(g, c_cols, block_m, mw, dtype, st);
 #define SK_GEMM(DT)                                                       \
   switch (block_m) {                                                      \
@@ -406,4 +409,34 @@ extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
   }
   if (dtype == kBF16) { SK_GEMM(kBF16) } else { SK_GEMM(kF16) }
 #undef SK_GEMM
+}
+}  // namespace sarathi_hip
+
+extern "C" int sarathi_moe_grouped_gemm(const void* a, const void* b, void* c,
+                                        const float* topk_weights,
+                                        const int32_t* sorted_token_ids,
+                                        const int32_t* expert_ids,
+                                        const int32_t* num_tokens_post_padded,
+                                        int64_t num_valid_tokens, int64_t sorted_len, int64_t n,
+                                        int64_t k, int64_t a_row_stride, int64_t b_expert_stride,
+                                        int64_t c_row_stride, int block_m, int top_k,
+                                        int epilogue, int b_layout, int dtype,
+                                        void* stream) {
+  return sarathi_hip::grouped_gemm(a, b, c, topk_weights, sorted_token_ids, expert_ids,
+                                   num_tokens_post_padded, num_valid_tokens, sorted_len, n, k,
+                                   a_row_stride, b_expert_stride, c_row_stride, block_m, top_k,
+                                   epilogue, b_layout, dtype, nullptr, stream);
+}
+
+extern "C" int sarathi_moe_grouped_gemm_riders(
+    const void* a, const void* b, void* c, const float* topk_weights,
+    const int32_t* sorted_token_ids, const int32_t* expert_ids,
+    const int32_t* num_tokens_post_padded, int64_t num_valid_tokens, int64_t sorted_len, int64_t n,
+    int64_t k, int64_t a_row_stride, int64_t b_expert_stride, int64_t c_row_stride, int block_m,
+    int top_k, int epilogue, int b_layout, int dtype, const int32_t* riders, void* stream) {
+  if (!riders) return SARATHI_ERR_INVALID_ARG;
+  return sarathi_hip::grouped_gemm(a, b, c, topk_weights, sorted_token_ids, expert_ids,
+                                   num_tokens_post_padded, num_valid_tokens, sorted_len, n, k,
+                                   a_row_stride, b_expert_stride, c_row_stride, block_m, top_k,
+                                   epilogue, b_layout, dtype, riders, stream);
 }

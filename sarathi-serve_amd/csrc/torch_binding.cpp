@@ -605,7 +605,8 @@ void moe_grouped_gemm(torch::Tensor& a, torch::Tensor& b, torch::Tensor& c,
                       torch::Tensor& topk_weights, torch::Tensor& sorted_token_ids,
                       torch::Tensor& expert_ids, torch::Tensor& num_tokens_post_padded,
                       int64_t num_valid_tokens, int64_t block_m, int64_t top_k,
-                      bool mul_routed_weight, bool b_packed, int64_t n, bool silu_and_mul) {
+                      bool mul_routed_weight, bool b_packed, int64_t n, bool silu_and_mul,
+                      const c10::optional<torch::Tensor>& riders) {
   const char* op = "moe_grouped_gemm";
   check_gpu(a, a, op, "A");
   check_gpu(b, a, op, "B");
@@ -655,18 +656,62 @@ void moe_grouped_gemm(torch::Tensor& a, torch::Tensor& b, torch::Tensor& c,
               op, ": routing tensors must be contiguous int32");
   TORCH_CHECK(block_m > 0 && expert_ids.numel() * block_m >= sorted_token_ids.numel(), op,
               ": expert_ids is too short for sorted_token_ids and block_m");
+  const int epilogue = silu_and_mul ? SARATHI_MOE_EPILOGUE_SILU_AND_MUL
+                       : mul_routed_weight ? SARATHI_MOE_EPILOGUE_ROUTED_WEIGHT
+                                           : SARATHI_MOE_EPILOGUE_NONE;
+  const int layout = b_packed ? SARATHI_MOE_B_PACKED : SARATHI_MOE_B_ROW_MAJOR;
   LaunchScope scope(a);
+  if (riders.has_value()) {
+    const torch::Tensor& r = *riders;
+    check_gpu(r, a, op, "riders");
+    TORCH_CHECK(r.scalar_type() == at::ScalarType::Int && r.is_contiguous() &&
+                    r.numel() * block_m >= sorted_token_ids.numel(),
+                op, ": riders must be contiguous int32 with one entry per slot block");
+    raise_on(sarathi_moe_grouped_gemm_riders(
+                 a.data_ptr(), b.data_ptr(), c.data_ptr(), topk_weights.data_ptr<float>(),
+                 sorted_token_ids.data_ptr<int32_t>(), expert_ids.data_ptr<int32_t>(),
+                 num_tokens_post_padded.data_ptr<int32_t>(), num_valid_tokens,
+                 sorted_token_ids.numel(), n, k, a.stride(0), expert_stride, c_cols, (int)block_m,
+                 (int)top_k, epilogue, layout, dtype_code(a, op), r.data_ptr<int32_t>(),
+                 scope.stream),
+             op);
+    return;
+  }
   raise_on(sarathi_moe_grouped_gemm(
                a.data_ptr(), b.data_ptr(), c.data_ptr(), topk_weights.data_ptr<float>(),
                sorted_token_ids.data_ptr<int32_t>(), expert_ids.data_ptr<int32_t>(),
                num_tokens_post_padded.data_ptr<int32_t>(), num_valid_tokens,
                sorted_token_ids.numel(), n, k, a.stride(0), expert_stride, c_cols, (int)block_m,
-               (int)top_k,
-               silu_and_mul ? SARATHI_MOE_EPILOGUE_SILU_AND_MUL
-                            : mul_routed_weight ? SARATHI_MOE_EPILOGUE_ROUTED_WEIGHT
-                                                : SARATHI_MOE_EPILOGUE_NONE,
-               b_packed ? SARATHI_MOE_B_PACKED : SARATHI_MOE_B_ROW_MAJOR, dtype_code(a, op),
-               scope.stream),
+               (int)top_k, epilogue, layout, dtype_code(a, op), scope.stream),
+           op);
+}
+
+// which 32-slot tiles of partly filled last blocks ride with which full blocks (input:
+// moe_align_block_size's outputs, greedy fill)
+void moe_plan_riders(torch::Tensor& sorted_token_ids, torch::Tensor& expert_ids,
+                     torch::Tensor& num_tokens_post_padded, int64_t num_valid_tokens,
+                     int64_t block_m, torch::Tensor& riders) {
+  const char* op = "moe_plan_riders";
+  check_gpu(sorted_token_ids, sorted_token_ids, op, "sorted_token_ids");
+  check_gpu(expert_ids, sorted_token_ids, op, "expert_ids");
+  check_gpu(num_tokens_post_padded, sorted_token_ids, op, "num_tokens_post_padded");
+  check_gpu(riders, sorted_token_ids, op, "riders");
+  TORCH_CHECK(sorted_token_ids.scalar_type() == at::ScalarType::Int &&
+                  expert_ids.scalar_type() == at::ScalarType::Int &&
+                  num_tokens_post_padded.scalar_type() == at::ScalarType::Int &&
+                  riders.scalar_type() == at::ScalarType::Int,
+              op, ": all tensors must be int32");
+  TORCH_CHECK(sorted_token_ids.is_contiguous() && expert_ids.is_contiguous() && riders.is_contiguous() &&
+                  num_tokens_post_padded.numel() >= 1,
+              op, ": tensors must be contiguous");
+  TORCH_CHECK(block_m > 0 && expert_ids.numel() * block_m >= sorted_token_ids.numel() &&
+                  riders.numel() * block_m >= sorted_token_ids.numel(),
+              op, ": expert_ids / riders are too short for sorted_token_ids and block_m");
+  LaunchScope scope(sorted_token_ids);
+  raise_on(sarathi_moe_plan_riders(sorted_token_ids.data_ptr<int32_t>(), expert_ids.data_ptr<int32_t>(),
+                                   num_tokens_post_padded.data_ptr<int32_t>(), num_valid_tokens,
+                                   sorted_token_ids.numel(), (int)block_m, riders.data_ptr<int32_t>(),
+                                   riders.numel(), scope.stream),
            op);
 }
 
@@ -784,5 +829,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         pybind11::arg("num_tokens_post_padded"), pybind11::arg("num_valid_tokens"),
         pybind11::arg("block_m"), pybind11::arg("top_k"), pybind11::arg("mul_routed_weight"),
         pybind11::arg("b_packed") = false, pybind11::arg("n") = 0,
-        pybind11::arg("silu_and_mul") = false);
+        pybind11::arg("silu_and_mul") = false, pybind11::arg("riders") = pybind11::none());
+  m.def("moe_plan_riders", &moe_plan_riders,
+        "for moe_grouped_gemm(riders=...): tiles of partly filled last blocks that full blocks take along",
+        pybind11::arg("sorted_token_ids"), pybind11::arg("expert_ids"),
+        pybind11::arg("num_tokens_post_padded"), pybind11::arg("num_valid_tokens"),
+        pybind11::arg("block_m"), pybind11::arg("riders"));
 }

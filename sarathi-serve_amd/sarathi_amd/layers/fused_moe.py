@@ -87,6 +87,14 @@ FUSE_SILU_AND_MUL = True
 # forward 2.69 ms greedy, 2.73 ms even; packed 2.66 / 2.67): a workgroup's time is mostly a fixed
 # cost per slot block, and an even fill has as many blocks as a greedy one.
 BALANCE_BLOCKS = False
+# Riders (moe_ops.moe_plan_riders): the few slots of an expert's partly filled last block are taken
+# along by the workgroups of its full blocks.  Row-major 16-bit weights at 256-slot blocks, from a
+# mean load of one block per expert (below that few experts have a full block to ride with, and
+# planning costs more than it saves).  Same bits either way.  Mixtral layer forward, MI355X, ms:
+#   tokens   512    768    1024   1536   2048   2560   3072   4096   6144   8192
+#   off      0.664  0.723  0.942  1.178  1.568  1.846  2.087  2.728  3.939  5.011
+#   on       0.702  0.789  0.917  1.167  1.399  1.829  2.059  2.540  3.751  4.909
+RIDERS = True
 CHUNK_SIZE = 64 * 1024     # tokens per pass, as in the reference (fused_moe.py:437)
 
 
@@ -170,7 +178,8 @@ def invoke_fused_moe_kernel(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor,
                             sorted_token_ids: torch.Tensor, expert_ids: torch.Tensor,
                             num_tokens_post_padded: torch.Tensor, mul_routed_weight: bool,
                             top_k: int, config: Dict[str, Any], compute_type=None,
-                            silu_and_mul: bool = False) -> None:
+                            silu_and_mul: bool = False,
+                            riders: Optional[torch.Tensor] = None) -> None:
     """Same argument list as the reference's launcher.  ``config["BLOCK_SIZE_M"]`` must be the block
     size ``sorted_token_ids`` was aligned with.  ``silu_and_mul=True`` (not in the reference):
     ``B`` is a gate/up projection ``[E, 2I, K]`` and ``C [.., I]`` receives
@@ -183,7 +192,8 @@ def invoke_fused_moe_kernel(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor,
     packed = isinstance(B, PackedExpertWeights)
     moe_ops.moe_grouped_gemm(A, B.data if packed else B, C, topk_weights, sorted_token_ids,
                              expert_ids, num_tokens_post_padded, topk_ids.numel(), block_m, top_k,
-                             bool(mul_routed_weight), packed, B.shape[1], bool(silu_and_mul))
+                             bool(mul_routed_weight), packed, B.shape[1], bool(silu_and_mul),
+                             riders)
 
 
 def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
@@ -243,17 +253,24 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
             sorted_ids = balance_blocks(sorted_ids, expert_ids, post_padded,
                                         config["BLOCK_SIZE_M"], E, n * topk,
                                         packed=isinstance(w1, PackedExpertWeights))
+        riders = None
+        if (RIDERS and config["BLOCK_SIZE_M"] == 256 and not is_f32 and n * topk >= 256 * E
+                and not isinstance(w1, PackedExpertWeights)
+                and not isinstance(w2, PackedExpertWeights)
+                and not (BALANCE_BLOCKS and config["BLOCK_SIZE_M"] >= 64)):
+            riders = torch.empty((expert_ids.numel(),), dtype=torch.int32, device=dev)
+            moe_ops.moe_plan_riders(sorted_ids, expert_ids, post_padded, n * topk, 256, riders)
         if fuse_act:
             invoke_fused_moe_kernel(cur_hidden, w1, c2, None, None, cur_w, cur_ids, sorted_ids,
                                     expert_ids, post_padded, False, topk, config,
-                                    silu_and_mul=True)
+                                    silu_and_mul=True, riders=riders)
         else:
             c1 = cache1[:n]
             invoke_fused_moe_kernel(cur_hidden, w1, c1, None, None, cur_w, cur_ids, sorted_ids,
-                                    expert_ids, post_padded, False, topk, config)
+                                    expert_ids, post_padded, False, topk, config, riders=riders)
             activation_ops.silu_and_mul(c2, c1.view(-1, N))
         invoke_fused_moe_kernel(c2, w2, c3, None, None, cur_w, cur_ids, sorted_ids, expert_ids,
-                                post_padded, True, 1, config)
+                                post_padded, True, 1, config, riders=riders)
         moe_ops.moe_sum(c3, out[begin:end])   # the reference's torch.sum(c3, dim=1, out=...)
     return out
 

@@ -30,9 +30,16 @@ moe_balance_blocks = _C.moe_balance_blocks
 # moe_gemm_slot_rows(block_m, b_packed): the rows_per_block that suits moe_grouped_gemm's kernel
 moe_gemm_slot_rows = _C.moe_gemm_slot_rows
 
+# moe_plan_riders(sorted_token_ids, expert_ids, num_tokens_post_padded, num_valid_tokens, block_m,
+#                 riders): fills `riders` (int32, one entry per slot block) for
+# moe_grouped_gemm(..., riders=riders): the few slots of an expert's partly filled last block are
+# multiplied by the workgroups of its full blocks instead of by workgroups of their own (row-major
+# 16-bit weights, block_m = 256; no counterpart in the reference)
+moe_plan_riders = _C.moe_plan_riders
+
 # moe_sum(input[tokens, top_k, hidden], out[tokens, hidden]): the torch.sum over the top-k expert
 # outputs that ends fused_experts (fused_moe.py:539-543)
 moe_sum = _C.moe_sum
 
-__all__ = ["moe_sum", "moe_balance_blocks", "moe_gemm_slot_rows", "topk_softmax", "moe_align_block_size", "topk_softmax_renorm",
+__all__ = ["moe_sum", "moe_plan_riders", "moe_balance_blocks", "moe_gemm_slot_rows", "topk_softmax", "moe_align_block_size", "topk_softmax_renorm",
            "moe_align_block_size_filled", "moe_grouped_gemm", "fused_topk_align", "grouped_topk"]

@@ -246,3 +246,36 @@ def test_new_entry_points_validate_arguments_without_gpu(lib):
     assert copy(dst=vp(q.value + 4)) == INVALID # unaligned
     assert copy(kib=5) == UNSUPPORTED           # no such launch shape
     assert copy(n=0) == OK
+
+
+def test_rider_entry_points_validate_arguments_without_gpu(lib):
+    """sarathi_moe_plan_riders and sarathi_moe_grouped_gemm_riders reject what the rider kernel does
+    not cover (other block sizes, packed weights, fp32) before anything is launched."""
+    i64, ci, vp = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p
+    buf = ctypes.create_string_buffer(256)
+    p = ctypes.cast(buf, vp)
+    null = vp(None)
+    INVALID, UNSUPPORTED, OK = -1, -2, 0
+
+    def plan(**kw):
+        return lib.sarathi_moe_plan_riders(
+            kw.get("ids", p), p, p, i64(kw.get("valid", 4)), i64(kw.get("len", 512)),
+            ci(kw.get("bm", 256)), kw.get("out", p), i64(kw.get("out_len", 2)), null)
+    assert plan(ids=null) == INVALID
+    assert plan(out=null) == INVALID
+    assert plan(out_len=1) == INVALID           # one entry per slot block
+    assert plan(valid=-1) == INVALID
+    assert plan(bm=128) == UNSUPPORTED
+    assert plan(len=0, out_len=0) == OK
+
+    def gemm(**kw):
+        return lib.sarathi_moe_grouped_gemm_riders(
+            kw.get("a", p), p, p, p, p, p, p, i64(kw.get("valid", 4)), i64(256),
+            i64(64), i64(64), i64(64), i64(64 * 128), i64(64), ci(kw.get("bm", 256)), ci(2),
+            ci(0), ci(kw.get("layout", 0)), ci(kw.get("dt", 2)), kw.get("riders", p), null)
+    assert gemm(riders=null) == INVALID
+    assert gemm(a=null) == INVALID
+    assert gemm(bm=128) == UNSUPPORTED
+    assert gemm(layout=1) == UNSUPPORTED
+    assert gemm(dt=0) == UNSUPPORTED
+    assert gemm(valid=0) == OK

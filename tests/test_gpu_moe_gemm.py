@@ -411,3 +411,90 @@ def test_gated_silu_epilogue_is_bit_identical_to_separate_kernels(ops, dev, dtyp
         ops.moe_ops.moe_grouped_gemm(A, packed.data, got2, w, s, e, p, T * k, BM, k, False, True,
                                      2 * I, True)
         assert torch.equal(got2, want)
+
+
+# ---------------------------------------------------------------- riders
+
+def _expected_riders(s, e, p, num_valid, bm):
+    """What sarathi_moe_plan_riders documents, from moe_align_block_size's outputs (numpy-free,
+    block by block)."""
+    s, e = s.tolist(), e.tolist()
+    live = min(int(p[0]), len(s)) // bm
+    out = [-1] * ((len(s) + bm - 1) // bm)
+    b = 0
+    while b < live:
+        last = b
+        while last + 1 < live and e[last + 1] == e[b]:
+            last += 1
+        valid = sum(1 for x in s[last * bm:(last + 1) * bm] if x < num_valid)
+        tiles = (valid + 31) // 32
+        if last > b and tiles <= last - b:
+            out[last] = -2
+            for j in range(tiles):
+                out[b + j] = last * bm + 32 * j
+        b = last + 1
+    return out
+
+
+@pytest.mark.parametrize("T,E,k", [(1100, 4, 2), (1024, 8, 2), (2048, 8, 2), (4096, 8, 2), (300, 8, 2),
+                                   (700, 2, 1), (5000, 16, 4)])
+def test_moe_plan_riders_matches_its_definition(ops, dev, T, E, k):
+    bm = 256
+    _, _, _, s, e, p = _route(T, E, k, bm, 31 * T + E)
+    want = _expected_riders(s, e, p, T * k, bm)
+    got = torch.full((e.numel(),), 99, dtype=torch.int32, device=dev)
+    ops.moe_ops.moe_plan_riders(s.to(dev), e.to(dev), p.to(dev), T * k, bm, got)
+    assert got.cpu().tolist() == want
+    if (T, E, k) in ((1100, 4, 2), (4096, 8, 2)):
+        assert any(x >= 0 for x in want) and any(x == -2 for x in want)   # the case exercises riders
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,k,N,K", [
+    (1100, 4, 2, 512, 256),     # 550 slots per expert: two full blocks and two tiles that ride
+    (1040, 8, 2, 520, 128),     # one full block and a few slots per expert; ragged N
+    (2100, 8, 2, 4104, 64),     # two K-stages only; 17 column blocks
+    (300, 8, 2, 512, 256),      # nothing to ride (single blocks)
+])
+def test_grouped_gemm_with_riders_same_bits(ops, dev, dtype, T, E, k, N, K):
+    """Row-major weights at 256-slot blocks: with the riders table the partly filled last blocks
+    are multiplied by the workgroups of the full blocks; every output is formed from the same
+    products in the same order, so all three epilogues give the same bits as without riders."""
+    bm = 256
+    _, w, ids, s, e, p = _route(T, E, k, bm, T + N)
+    g = gen(K + T)
+    A = randn((T, K), g, dtype, std=0.5).to(dev)
+    Bw = randn((E, N, K), g, dtype, std=0.5).to(dev)
+    sd, ed, pd, wd = s.to(dev), e.to(dev), p.to(dev), w.to(dev)
+    riders = torch.empty((e.numel(),), dtype=torch.int32, device=dev)
+    ops.moe_ops.moe_plan_riders(sd, ed, pd, T * k, bm, riders)
+    for mul, silu in ((False, False), (True, False), (False, True)):
+        cols = N // 2 if silu else N
+        base = torch.full((T, k, cols), 7.0, dtype=dtype, device=dev)
+        with_r = torch.full((T, k, cols), -3.0, dtype=dtype, device=dev)
+        ops.moe_ops.moe_grouped_gemm(A, Bw, base, wd, sd, ed, pd, T * k, bm, k, mul, False, N, silu)
+        ops.moe_ops.moe_grouped_gemm(A, Bw, with_r, wd, sd, ed, pd, T * k, bm, k, mul, False, N, silu,
+                                     riders)
+        assert torch.equal(with_r, base), (mul, silu)
+    # the table is refused where the kernel that reads it does not run
+    with pytest.raises(RuntimeError):
+        ops.moe_ops.moe_grouped_gemm(A, Bw, base, wd, sd, ed, pd, T * k, 128, k, False, False, N, False,
+                                     riders)
+
+
+def test_fused_moe_same_bits_with_and_without_riders(ops, dev, monkeypatch):
+    import importlib
+    from sarathi_amd import layers
+    fm = importlib.import_module("sarathi_amd.layers.fused_moe")   # the module, not the function
+    T, E, k, H, I = 1100, 4, 2, 512, 1024
+    g = gen(5)
+    x = randn((T, H), g, torch.bfloat16, std=0.5).to(dev)
+    w1 = randn((E, 2 * I, H), g, torch.bfloat16, std=0.05).to(dev)
+    w2 = randn((E, H, I), g, torch.bfloat16, std=0.05).to(dev)
+    logits = torch.randn((T, E), generator=g, dtype=torch.float32).to(dev)
+    cfg = {"BLOCK_SIZE_M": 256}
+    monkeypatch.setattr(fm, "RIDERS", False)
+    base = layers.fused_moe(x, w1, w2, logits, k, True, override_config=cfg)
+    monkeypatch.setattr(fm, "RIDERS", True)
+    got = layers.fused_moe(x, w1, w2, logits, k, True, override_config=cfg)
+    assert torch.equal(got, base)
