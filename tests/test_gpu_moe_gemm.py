@@ -482,6 +482,42 @@ def test_grouped_gemm_with_riders_same_bits(ops, dev, dtype, T, E, k, N, K):
                                      riders)
 
 
+@pytest.mark.parametrize("loads", [
+    (1024 + 33, 257, 0, 255, 512, 31),          # 2 tiles on 4 full blocks; 1 slot on one; exact blocks
+    (8 * 256 + 255, 0, 0, 1),                   # a last block of eight tiles, all riding
+    (8 * 256 + 256, 3 * 256 + 97, 2 * 256 + 65),  # no partial block; four tiles > three blocks; 3 > 2
+    (256 + 32, 256 + 33, 512 + 64, 512 + 65),   # either side of the tile and block-count limits
+])
+def test_riders_with_chosen_expert_loads(ops, dev, loads):
+    """Expert loads picked to sit on the limits of the plan (a tile more than there are full blocks,
+    a last block that is full, empty experts, one slot): the table is the documented one and the
+    GEMM has the same bits with it."""
+    bm, E, N, K = 256, len(loads), 520, 192
+    g = gen(sum(loads))
+    order = torch.cat([torch.full((n,), x, dtype=torch.int32) for x, n in enumerate(loads)])
+    ids = order[torch.randperm(order.numel(), generator=g)].view(-1, 1)
+    T = ids.numel()
+    n = T + E * (bm - 1)
+    s = torch.full((n,), T, dtype=torch.int32)
+    e = torch.zeros(((n + bm - 1) // bm,), dtype=torch.int32)
+    p = torch.zeros((1,), dtype=torch.int32)
+    c_oracle.moe_align_block_size(ids, E, bm, s, e, p)
+    sd, ed, pd = s.to(dev), e.to(dev), p.to(dev)
+    riders = torch.full((e.numel(),), 99, dtype=torch.int32, device=dev)
+    ops.moe_ops.moe_plan_riders(sd, ed, pd, T, bm, riders)
+    assert riders.cpu().tolist() == _expected_riders(s, e, p, T, bm)
+    A = randn((T, K), g, torch.bfloat16, std=0.5).to(dev)
+    Bw = randn((E, N, K), g, torch.bfloat16, std=0.5).to(dev)
+    wd = torch.rand((T, 1), generator=g).to(dev)
+    for mul, silu in ((True, False), (False, True)):
+        cols = N // 2 if silu else N
+        base = torch.full((T, 1, cols), 7.0, dtype=torch.bfloat16, device=dev)
+        with_r = torch.full((T, 1, cols), -3.0, dtype=torch.bfloat16, device=dev)
+        ops.moe_ops.moe_grouped_gemm(A, Bw, base, wd, sd, ed, pd, T, bm, 1, mul, False, N, silu)
+        ops.moe_ops.moe_grouped_gemm(A, Bw, with_r, wd, sd, ed, pd, T, bm, 1, mul, False, N, silu, riders)
+        assert torch.equal(with_r, base), (mul, silu)
+
+
 def test_fused_moe_same_bits_with_and_without_riders(ops, dev, monkeypatch):
     import importlib
     from sarathi_amd import layers
