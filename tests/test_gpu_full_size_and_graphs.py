@@ -293,3 +293,44 @@ def test_mixtral_expert_gemms_full_size(ops, dev):
     ops.activation_ops.silu_and_mul(act, plain)
     assert torch.equal(run(x, w1, False, True), act)
     assert torch.equal(run(x, packed_w1, True, True), act)
+
+
+def test_fused_moe_with_riders_under_hip_graph_capture(ops, dev, monkeypatch):
+    """The riders table is planned on the device from the batch's own routing: a captured
+    fused_moe replayed on new activations and router logits (other expert loads, other riders)
+    equals the eager layer without riders, bit for bit, on every replay."""
+    import importlib
+    from sarathi_amd import layers
+    fm = importlib.import_module("sarathi_amd.layers.fused_moe")   # the module, not the function
+    T, E, k, H, I = 1100, 4, 2, 256, 512
+    cfg = {"BLOCK_SIZE_M": 256}
+    g = gen(23)
+    w1 = randn((E, 2 * I, H), g, std=H ** -0.5).to(dev)
+    w2 = randn((E, H, I), g, std=I ** -0.5).to(dev)
+    batches = []
+    for i in range(4):
+        x = randn((T, H), g, std=0.5).to(dev)
+        logits = torch.randn((T, E), generator=g, dtype=torch.float32)
+        logits[:, i % E] += 0.4 * i          # shift the loads: other blocks end up short
+        batches.append((x, logits.to(dev)))
+    monkeypatch.setattr(fm, "RIDERS", False)
+    want = [layers.fused_moe(x, w1, w2, lg, k, True, override_config=cfg) for x, lg in batches]
+    monkeypatch.setattr(fm, "RIDERS", True)
+    xs, ls = batches[0][0].clone(), batches[0][1].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        layers.fused_moe(xs, w1, w2, ls, k, True, override_config=cfg)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = layers.fused_moe(xs, w1, w2, ls, k, True, override_config=cfg)
+    for (x, lg), expect in zip(batches + batches[:1], want + want[:1]):
+        xs.copy_(x)
+        ls.copy_(lg)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, expect)
+        _ = (x.float().sum() + lg.sum()).item()
