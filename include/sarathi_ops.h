@@ -386,8 +386,10 @@ int sarathi_moe_balance_blocks(const int32_t* sorted_in, int32_t* sorted_out,
  * last block rides when it holds at most as many 32-slot tiles as the expert has full blocks.
  * sarathi_moe_grouped_gemm_riders is sarathi_moe_grouped_gemm with that table: row-major weights,
  * block_m = 256, bfloat16 / float16 (anything else: SARATHI_ERR_UNSUPPORTED); same results bit
- * for bit (a slot's dot products do not depend on which workgroup forms them).  The sorted ids
- * must be in moe_align_block_size's greedy order (not rewritten by sarathi_moe_balance_blocks).
+ * for bit (a slot's dot products do not depend on which workgroup forms them).  A launch so
+ * small that the plain kernel takes 128-wide column blocks to fill the chip runs that kernel and
+ * ignores the table.  The sorted ids must be in moe_align_block_size's greedy order (not rewritten
+ * by sarathi_moe_balance_blocks).
  */
 int sarathi_moe_plan_riders(const int32_t* sorted_token_ids, const int32_t* expert_ids,
                             const int32_t* num_tokens_post_padded, int64_t num_valid_tokens,

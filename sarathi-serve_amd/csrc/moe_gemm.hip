@@ -305,6 +305,7 @@ static int launch_moe_gemm(const MoeGemmArgs& g, int epilogue, bool packed, hipS
 // moe_gemm_wide.hip: row-major weights at 64-, 128- and 256-slot blocks, four waves
 int launch_moe_gemm_wide(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, int dtype,
                          hipStream_t st);
+bool moe_gemm_wide_takes_narrow_blocks(int64_t out_cols, int m_blocks, int block_m, int epilogue);
 // moe_gemm_rider.hip: row-major weights at 256-slot blocks, with riders
 int launch_moe_gemm_rider(MoeGemmArgs g, int64_t out_cols, int epilogue, int dtype,
                          const int32_t* ride, hipStream_t st);
@@ -398,7 +399,10 @@ static int grouped_gemm(const void* a, const void* b, void* c, const float* topk
   const int mw = epilogue;
   // row-major weights run the four-wave kernel of moe_gemm_wide.hip from 64-slot blocks on (32-slot
   // wave tiles for decode-size batches, 128 x 128 wave tiles at 256-slot blocks)
-  if (ride) return launch_moe_gemm_rider(g, c_cols, mw, dtype, ride, st);
+  // riders are an optimisation (the plain kernels compute every block themselves): a launch so
+  // small that the plain kernel would take 128-wide column blocks to fill the chip keeps those
+  if (ride && !moe_gemm_wide_takes_narrow_blocks(c_cols, g.m_blocks, block_m, mw))
+    return launch_moe_gemm_rider(g, c_cols, mw, dtype, ride, st);
   if (!packed && block_m >= 64) return launch_moe_gemm_wide(g, c_cols, block_m, mw, dtype, st);
 #define SK_GEMM(DT)                                                       \
   switch (block_m) {                                                      \

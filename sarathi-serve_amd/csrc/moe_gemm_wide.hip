@@ -325,17 +325,21 @@ static int launch_wide_epilogue(MoeGemmArgs g, int64_t out_cols, int epilogue, h
 
 // Entry used by sarathi_moe_grouped_gemm for row-major weights at 64-, 128- and 256-slot blocks.  `g`
 // is complete except for n_blocks, which depends on the epilogue and the column-block width.
+// Column blocks of 256 unless that leaves compute units short of workgroups.  Measured on the
+// Mixtral projections: at 256-slot blocks (one workgroup per compute unit) 128-wide blocks are
+// 1-12 % faster while the wide launch has fewer than 256 workgroups and 20 % slower from there
+// on; at 64-slot blocks (two to three per compute unit) they are faster up to 896 workgroups
+// (16-64 tokens: gate/up projection 0.333 -> 0.326 ms, down projection 0.205 -> 0.178 ms) and
+// slower at 1792 (256 tokens).
+bool moe_gemm_wide_takes_narrow_blocks(int64_t out_cols, int m_blocks, int block_m, int epilogue) {
+  const int64_t cols_wide = epilogue == kEpiGatedSilu ? 128 : 256;
+  const int64_t wide_blocks = (out_cols + cols_wide - 1) / cols_wide * m_blocks;
+  return block_m != 128 && wide_blocks < (block_m == 256 ? 256 : 1024);
+}
+
 int launch_moe_gemm_wide(MoeGemmArgs g, int64_t out_cols, int block_m, int epilogue, int dtype,
                          hipStream_t st) {
-  // Column blocks of 256 unless that leaves compute units short of workgroups.  Measured on the
-  // Mixtral projections: at 256-slot blocks (one workgroup per compute unit) 128-wide blocks are
-  // 1-12 % faster while the wide launch has fewer than 256 workgroups and 20 % slower from there
-  // on; at 64-slot blocks (two to three per compute unit) they are faster up to 896 workgroups
-  // (16-64 tokens: gate/up projection 0.333 -> 0.326 ms, down projection 0.205 -> 0.178 ms) and
-  // slower at 1792 (256 tokens).
-  const int64_t cols_wide = epilogue == kEpiGatedSilu ? 128 : 256;
-  const int64_t wide_blocks = (out_cols + cols_wide - 1) / cols_wide * g.m_blocks;
-  const bool narrow = wide_blocks < (block_m == 256 ? 256 : 1024);
+  const bool narrow = moe_gemm_wide_takes_narrow_blocks(out_cols, g.m_blocks, block_m, epilogue);
 #define SK_PICK(DT)                                                                               \
   if (block_m == 256)                                                                             \
     return narrow ? launch_wide_epilogue<DT, 128, 256>(g, out_cols, epilogue, st)                 \

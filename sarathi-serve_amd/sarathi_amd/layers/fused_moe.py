@@ -89,11 +89,12 @@ FUSE_SILU_AND_MUL = True
 BALANCE_BLOCKS = False
 # Riders (moe_ops.moe_plan_riders): the few slots of an expert's partly filled last block are taken
 # along by the workgroups of its full blocks.  Row-major 16-bit weights at 256-slot blocks, from a
-# mean load of one block per expert (below that few experts have a full block to ride with, and
-# planning costs more than it saves).  Same bits either way.  Mixtral layer forward, MI355X, ms:
+# mean load of half a block per expert (below that an expert with more than one block is rare, and
+# planning costs a launch: about 1 % of the layer).  Same bits either way.  Mixtral layer forward,
+# N(0, 1) router logits, MI355X, ms:
 #   tokens   512    768    1024   1536   2048   2560   3072   4096   6144   8192
-#   off      0.664  0.723  0.942  1.178  1.568  1.846  2.087  2.728  3.939  5.011
-#   on       0.702  0.789  0.917  1.167  1.399  1.829  2.059  2.540  3.751  4.909
+#   off      0.654  0.717  0.942  1.178  1.568  1.846  2.087  2.728  3.939  5.011
+#   on       0.657  0.726  0.917  1.167  1.399  1.829  2.059  2.540  3.751  4.909
 RIDERS = True
 CHUNK_SIZE = 64 * 1024     # tokens per pass, as in the reference (fused_moe.py:437)
 
@@ -254,7 +255,7 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
                                         config["BLOCK_SIZE_M"], E, n * topk,
                                         packed=isinstance(w1, PackedExpertWeights))
         riders = None
-        if (RIDERS and config["BLOCK_SIZE_M"] == 256 and not is_f32 and n * topk >= 256 * E
+        if (RIDERS and config["BLOCK_SIZE_M"] == 256 and not is_f32 and 2 * n * topk >= 256 * E
                 and not isinstance(w1, PackedExpertWeights)
                 and not isinstance(w2, PackedExpertWeights)
                 and not (BALANCE_BLOCKS and config["BLOCK_SIZE_M"] >= 64)):
