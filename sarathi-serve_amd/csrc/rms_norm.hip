@@ -303,7 +303,8 @@ static int launch_rms(void* out, void* in, const void* w, float eps, int64_t T, 
   // Fused op on rows of 257..512 vectors outside that range: two or three rows per one-wave
   // workgroup where the row count makes that come out even over the compute units.  (The plain
   // norm gains nothing from several rows per wave, from holding its stores back, or from two
-  // waves per row: 7.1, 7.3, 7.5, 7.7 us at 2304 x 4096.)
+  // waves per row: 7.1, 7.3, 7.5, 7.7 us at 2304 x 4096; nor from workgroups of two, three or four
+  // independent one-row waves: 7.6, 7.4, 8.6 us against 7.4 for that kernel with one wave.)
   if (FUSED && nvec > 256 && nvec <= 512 && out_stride / N <= 0xffffffffLL &&
       in_stride / N <= 0xffffffffLL) {
     const int rows_per_wg = pick_rows_per_workgroup(T, 3);
