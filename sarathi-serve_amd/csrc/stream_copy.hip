@@ -21,6 +21,8 @@ __global__ __launch_bounds__(64) void stream_copy_kernel(void* __restrict__ dst,
   u32x4 v[VPL];
 #pragma unroll
   for (int j = 0; j < VPL; ++j) v[j] = buf_load16<kStreamLoad>(ri, off0 + j * 1024u);
+  // left alone, the scheduler starts storing after about ten loads and issues the rest one by one
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int j = 0; j < VPL; ++j) buf_store16<kStreamStore>(ro, off0 + j * 1024u, v[j]);
 }
