@@ -156,8 +156,9 @@ def main():
     ap.add_argument("--moe-riders", choices=["on", "off"], default="on",
                     help="moe section, row-major weights at 256-slot blocks: the slots of an expert's "
                          "partly filled last block ride with the workgroups of its full blocks "
-                         "(moe_ops.moe_plan_riders; the library's default) or get workgroups of "
-                         "their own")
+                         "and the other experts' slots are spread evenly over their blocks "
+                         "(moe_ops.moe_plan_blocks; the library's default), or blocks stay as "
+                         "moe_align_block_size fills them")
     ap.add_argument("--moe-block-m", type=int, default=0,
                     help="moe section: slot-block size of the grouped GEMMs (0 = the library's choice)")
     args = ap.parse_args()
@@ -676,7 +677,9 @@ def main():
             rd = None
             if args.moe_riders == "on" and label == "row_major" and bm == 256 and args.moe_balance != "on":
                 rd = torch.empty((e_ids.numel(),), dtype=torch.int32, device=dev)
-                MOE.moe_plan_riders(s_ids, e_ids, p_pad, Tn * k, bm, rd)
+                planned = torch.empty_like(s_ids)     # what fused_experts does: riders, even fill for the rest
+                MOE.moe_plan_blocks(s_ids, planned, e_ids, p_pad, E, bm, Tn * k, rd)
+                s_ids = planned
             ms1 = timeit_ms(lambda: MOE.moe_grouped_gemm(
                 x, b1, c1, tw_m, s_ids, e_ids, p_pad, Tn * k, bm, k, False, pk, 2 * I, False, rd))
             ms_act = timeit_ms(lambda: ACT.silu_and_mul(c2, c1.view(-1, 2 * I)))
@@ -699,7 +702,7 @@ def main():
                      "warm in L2/MALL as far as they fit)"
                      % (args.moe_data, args.moe_routing,
                         "filled evenly per expert" if args.moe_balance == "on"
-                        else "filled greedily, riders" if args.moe_riders == "on" else "filled greedily"),
+                        else "planned per expert (riders or even fill)" if args.moe_riders == "on" else "filled greedily"),
             "peak": "2500 TFLOP/s dense bf16 MFMA; 8 TB/s HBM",
             "fused_moe_forward_row_major": forward, "at_4096_tokens": gemms}
 

@@ -404,6 +404,24 @@ int sarathi_moe_grouped_gemm_riders(const void* a, const void* b, void* c, const
                                     const int32_t* riders, void* stream);
 
 /*
+ * No counterpart in the reference: sarathi_moe_plan_riders and sarathi_moe_balance_blocks in one
+ * launch, the choice made per expert (block_m = 256 only, SARATHI_ERR_UNSUPPORTED otherwise).  An
+ * expert whose last block holds at most as many 32-slot tiles as the expert has full blocks keeps
+ * moe_align_block_size's layout in `sorted_out` and gets riders; every other expert's slots are
+ * spread evenly over the two 128-slot halves of each of its blocks (what
+ * sarathi_moe_balance_blocks does with granule 32 and rows_per_block 2: a block costs the GEMM as
+ * much as its fuller half) and its entries of `riders` are -1.  `sorted_out` (same length as
+ * `sorted_in`, not the same memory) and `riders` (one int32 per slot block, at least
+ * ceil(sorted_len / block_m)) then go to sarathi_moe_grouped_gemm_riders together with the
+ * unchanged expert_ids and num_tokens_post_padded.  `pad_value` is the padding id
+ * (num_valid_tokens).  Same GEMM results bit for bit.
+ */
+int sarathi_moe_plan_blocks(const int32_t* sorted_in, int32_t* sorted_out, const int32_t* expert_ids,
+                            const int32_t* num_tokens_post_padded, int64_t sorted_len,
+                            int num_experts, int block_m, int pad_value, int32_t* riders,
+                            int64_t riders_len, void* stream);
+
+/*
  * No counterpart in the reference: how many equal ranges of a slot block the waves of the
  * sarathi_moe_grouped_gemm kernel for (block_m, b_layout) split between them (1 or 2; each range
  * is swept by its own waves, 32 slots at a time, and ranges without a valid slot in a tile are

@@ -84,7 +84,100 @@ __global__ __launch_bounds__(256) void moe_balance_blocks_kernel(
   }
 }
 
+// The two remedies for a partly filled last block, chosen per expert (256-slot blocks, the
+// four-wave kernel with riders).  An expert whose last block holds at most as many 32-slot tiles
+// as it has full blocks keeps the greedy layout and gets riders: tile j of the last block goes
+// along with the expert's j-th block, and the last block is skipped.  Any other expert gets the
+// even fill over the two 128-slot wave rows of each of its blocks and no riders.  Same
+// workgroup layout as the kernel above: one per expert plus one for the tail of both outputs.
+// `ride` as moe_gemm_rider.hip reads it: -2 skip the block, >= 0 first slot of the tile that
+// rides with this block, -1 neither.
+__global__ __launch_bounds__(256) void moe_plan_blocks_kernel(
+    const int32_t* __restrict__ sorted_in, int32_t* __restrict__ sorted_out,
+    const int32_t* __restrict__ expert_ids, const int32_t* __restrict__ post_pad,
+    int64_t sorted_len, int num_experts, int pad_value, int32_t* __restrict__ ride,
+    int ride_len) {
+  constexpr int block = 256, granule = 32, rows = 2;
+  __shared__ int first_blk, last_blk, valid_last;
+  const int tid = threadIdx.x;
+  int64_t end = *post_pad;
+  if (end > sorted_len) end = sorted_len;
+  const int nblk_total = (int)(end / block);
+  if ((int)blockIdx.x == num_experts) {
+    for (int64_t i = end + tid; i < sorted_len; i += 256) sorted_out[i] = pad_value;
+    for (int b = nblk_total + tid; b < ride_len; b += 256) ride[b] = -1;
+    return;
+  }
+  const int e = blockIdx.x;
+  if (tid == 0) {
+    first_blk = nblk_total;
+    last_blk = -1;
+    valid_last = 0;
+  }
+  __syncthreads();
+  int lo = nblk_total, hi = -1;
+  for (int b = tid; b < nblk_total; b += 256)
+    if (expert_ids[b] == e) {
+      lo = b < lo ? b : lo;
+      hi = b > hi ? b : hi;
+    }
+  if (hi >= 0) {
+    atomicMin(&first_blk, lo);
+    atomicMax(&last_blk, hi);
+  }
+  __syncthreads();
+  const int b0 = first_blk, b1 = last_blk;
+  if (b1 < 0) return;  // the expert has no block (uniform)
+  const int nb = b1 - b0 + 1;
+  const int64_t base = (int64_t)b0 * block;
+  int c = 0;
+  for (int i = tid; i < block; i += 256) c += sorted_in[(int64_t)b1 * block + i] != pad_value;
+  if (c) atomicAdd(&valid_last, c);
+  __syncthreads();
+  const int tiles_last = (valid_last + granule - 1) / granule;
+  if (nb > 1 && tiles_last <= nb - 1) {  // riders, greedy layout kept
+    for (int i = tid; i < nb * block; i += 256) sorted_out[base + i] = sorted_in[base + i];
+    for (int b = tid; b < nb; b += 256)
+      ride[b0 + b] = b == nb - 1 ? -2 : b < tiles_last ? b1 * block + granule * b : -1;
+    return;
+  }
+  for (int b = tid; b < nb; b += 256) ride[b0 + b] = -1;
+  const int cnt = (nb - 1) * block + valid_last;
+  const int range = block / rows, ranges = nb * rows;
+  const int tiles = (cnt + granule - 1) / granule;
+  const int base_tiles = tiles / ranges, extra = tiles - base_tiles * ranges;
+  for (int i = tid; i < nb * block; i += 256) {
+    const int j = i / range, off = i - j * range;
+    const int mine = (base_tiles + (j < extra ? 1 : 0)) * granule;
+    const int before = (j * base_tiles + (j < extra ? j : extra)) * granule;
+    const int r = before + off;
+    sorted_out[base + i] = (off < mine && r < cnt) ? sorted_in[base + r] : pad_value;
+  }
+}
+
 }  // namespace sarathi_hip
+
+extern "C" int sarathi_moe_plan_blocks(const int32_t* sorted_in, int32_t* sorted_out,
+                                       const int32_t* expert_ids,
+                                       const int32_t* num_tokens_post_pad, int64_t sorted_len,
+                                       int num_experts, int block_m, int pad_value,
+                                       int32_t* riders, int64_t riders_len, void* stream) {
+  using namespace sarathi_hip;
+  if (sorted_len < 0 || num_experts <= 0 || block_m <= 0 || riders_len < 0)
+    return SARATHI_ERR_INVALID_ARG;
+  if (block_m != 256) return SARATHI_ERR_UNSUPPORTED;
+  if (riders_len < (sorted_len + block_m - 1) / block_m) return SARATHI_ERR_INVALID_ARG;
+  if (sorted_len == 0) return SARATHI_OK;
+  if (!sorted_in || !sorted_out || !expert_ids || !num_tokens_post_pad || !riders ||
+      sorted_in == sorted_out)
+    return SARATHI_ERR_INVALID_ARG;
+  if (num_experts > 1024 || sorted_len > 0x7fffffffLL || riders_len > 0x7fffffffLL)
+    return SARATHI_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(moe_plan_blocks_kernel, dim3((unsigned)num_experts + 1), dim3(256), 0,
+                     (hipStream_t)stream, sorted_in, sorted_out, expert_ids, num_tokens_post_pad,
+                     sorted_len, num_experts, pad_value, riders, (int)riders_len);
+  return launch_status();
+}
 
 extern "C" int sarathi_moe_balance_blocks(const int32_t* sorted_in, int32_t* sorted_out,
                                           const int32_t* expert_ids,

@@ -715,6 +715,39 @@ void moe_plan_riders(torch::Tensor& sorted_token_ids, torch::Tensor& expert_ids,
            op);
 }
 
+// per expert: riders (greedy layout kept) or even fill of its blocks (input: moe_align_block_size's
+// outputs)
+void moe_plan_blocks(torch::Tensor& sorted_in, torch::Tensor& sorted_out, torch::Tensor& expert_ids,
+                     torch::Tensor& num_tokens_post_pad, int64_t num_experts, int64_t block_m,
+                     int64_t pad_value, torch::Tensor& riders) {
+  const char* op = "moe_plan_blocks";
+  check_gpu(sorted_in, sorted_in, op, "sorted_in");
+  check_gpu(sorted_out, sorted_in, op, "sorted_out");
+  check_gpu(expert_ids, sorted_in, op, "expert_ids");
+  check_gpu(num_tokens_post_pad, sorted_in, op, "num_tokens_post_pad");
+  check_gpu(riders, sorted_in, op, "riders");
+  TORCH_CHECK(sorted_in.scalar_type() == at::ScalarType::Int && sorted_out.scalar_type() == at::ScalarType::Int &&
+                  expert_ids.scalar_type() == at::ScalarType::Int &&
+                  num_tokens_post_pad.scalar_type() == at::ScalarType::Int &&
+                  riders.scalar_type() == at::ScalarType::Int,
+              op, ": all tensors must be int32");
+  TORCH_CHECK(sorted_in.is_contiguous() && sorted_out.is_contiguous() && expert_ids.is_contiguous() &&
+                  riders.is_contiguous() && sorted_in.numel() == sorted_out.numel() &&
+                  num_tokens_post_pad.numel() >= 1,
+              op, ": tensors must be contiguous, sorted_in and sorted_out equally long");
+  TORCH_CHECK(sorted_in.data_ptr() != sorted_out.data_ptr(), op, ": cannot run in place");
+  TORCH_CHECK(block_m > 0 && num_experts > 0 &&
+                  expert_ids.numel() * block_m >= sorted_in.numel() &&
+                  riders.numel() * block_m >= sorted_in.numel(),
+              op, ": expert_ids / riders are too short for sorted_in and block_m");
+  LaunchScope scope(sorted_in);
+  raise_on(sarathi_moe_plan_blocks(sorted_in.data_ptr<int32_t>(), sorted_out.data_ptr<int32_t>(),
+                                   expert_ids.data_ptr<int32_t>(), num_tokens_post_pad.data_ptr<int32_t>(),
+                                   sorted_in.numel(), (int)num_experts, (int)block_m, (int)pad_value,
+                                   riders.data_ptr<int32_t>(), riders.numel(), scope.stream),
+           op);
+}
+
 // even fill of every expert's slot blocks (input: moe_align_block_size's outputs)
 void moe_balance_blocks(torch::Tensor& sorted_in, torch::Tensor& sorted_out, torch::Tensor& expert_ids,
                         torch::Tensor& num_tokens_post_pad, int64_t num_experts, int64_t block_size,
@@ -830,6 +863,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         pybind11::arg("block_m"), pybind11::arg("top_k"), pybind11::arg("mul_routed_weight"),
         pybind11::arg("b_packed") = false, pybind11::arg("n") = 0,
         pybind11::arg("silu_and_mul") = false, pybind11::arg("riders") = pybind11::none());
+  m.def("moe_plan_blocks", &moe_plan_blocks,
+        "per expert: riders for its last block, or its slots spread evenly over its blocks",
+        pybind11::arg("sorted_in"), pybind11::arg("sorted_out"), pybind11::arg("expert_ids"),
+        pybind11::arg("num_tokens_post_pad"), pybind11::arg("num_experts"), pybind11::arg("block_m"),
+        pybind11::arg("pad_value"), pybind11::arg("riders"));
   m.def("moe_plan_riders", &moe_plan_riders,
         "for moe_grouped_gemm(riders=...): tiles of partly filled last blocks that full blocks take along",
         pybind11::arg("sorted_token_ids"), pybind11::arg("expert_ids"),

@@ -88,14 +88,20 @@ FUSE_SILU_AND_MUL = True
 # cost per slot block, and an even fill has as many blocks as a greedy one.
 BALANCE_BLOCKS = False
 # Riders (moe_ops.moe_plan_riders): the few slots of an expert's partly filled last block are taken
-# along by the workgroups of its full blocks.  Row-major 16-bit weights at 256-slot blocks, from a
-# mean load of half a block per expert (below that an expert with more than one block is rare, and
-# planning costs a launch: about 1 % of the layer).  Same bits either way.  Mixtral layer forward,
-# N(0, 1) router logits, MI355X, ms:
-#   tokens   512    768    1024   1536   2048   2560   3072   4096   6144   8192
-#   off      0.654  0.717  0.942  1.178  1.568  1.846  2.087  2.728  3.939  5.011
-#   on       0.657  0.726  0.917  1.167  1.399  1.829  2.059  2.540  3.751  4.909
+# along by the workgroups of its full blocks.  Row-major 16-bit weights at 256-slot blocks.
 RIDERS = True
+# ... and the experts whose last block cannot ride (more 32-slot tiles in it than the expert has
+# full blocks) get their slots spread evenly over the two 128-slot halves of each of their blocks:
+# a block costs the GEMM as much as its fuller half (moe_ops.moe_plan_blocks: both in one launch).
+# Planned from a mean load of half a block per expert: below that the even fill wakes the second
+# pair of waves of every workgroup for a tile or two and costs 2-10 %.  Same bits either way.
+# Mixtral layer forward, N(0, 1) router logits, MI355X, ms (off: neither; on: both, the default;
+# riders: RIDERS_EVEN_REST = False):
+#   tokens   512    640    1024   1280   1536   2048   2560   3072   4096   6144
+#   off      0.651  0.680  0.934  1.130  1.183  1.558  1.860  2.097  2.731  3.959
+#   on       0.631  0.664  0.907  1.035  1.112  1.421  1.810  2.065  2.569  3.777
+#   riders   0.651  0.685  0.911  1.121  1.181  1.415  1.843  2.069  2.568  3.772
+RIDERS_EVEN_REST = True
 CHUNK_SIZE = 64 * 1024     # tokens per pass, as in the reference (fused_moe.py:437)
 
 
@@ -260,7 +266,13 @@ def fused_experts(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tenso
                 and not isinstance(w2, PackedExpertWeights)
                 and not (BALANCE_BLOCKS and config["BLOCK_SIZE_M"] >= 64)):
             riders = torch.empty((expert_ids.numel(),), dtype=torch.int32, device=dev)
-            moe_ops.moe_plan_riders(sorted_ids, expert_ids, post_padded, n * topk, 256, riders)
+            if RIDERS_EVEN_REST:
+                planned = torch.empty_like(sorted_ids)
+                moe_ops.moe_plan_blocks(sorted_ids, planned, expert_ids, post_padded, E, 256,
+                                        n * topk, riders)
+                sorted_ids = planned
+            else:
+                moe_ops.moe_plan_riders(sorted_ids, expert_ids, post_padded, n * topk, 256, riders)
         if fuse_act:
             invoke_fused_moe_kernel(cur_hidden, w1, c2, None, None, cur_w, cur_ids, sorted_ids,
                                     expert_ids, post_padded, False, topk, config,

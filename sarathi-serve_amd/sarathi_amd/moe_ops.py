@@ -36,10 +36,15 @@ moe_gemm_slot_rows = _C.moe_gemm_slot_rows
 # multiplied by the workgroups of its full blocks instead of by workgroups of their own (row-major
 # 16-bit weights, block_m = 256; no counterpart in the reference)
 moe_plan_riders = _C.moe_plan_riders
+# moe_plan_blocks(sorted_in, sorted_out, expert_ids, num_tokens_post_pad, num_experts, block_m,
+#                 pad_value, riders): moe_plan_riders and moe_balance_blocks in one launch, chosen per
+# expert: riders where the last block's tiles fit onto the expert's full blocks (layout kept), an
+# even fill of the expert's blocks otherwise (block_m = 256)
+moe_plan_blocks = _C.moe_plan_blocks
 
 # moe_sum(input[tokens, top_k, hidden], out[tokens, hidden]): the torch.sum over the top-k expert
 # outputs that ends fused_experts (fused_moe.py:539-543)
 moe_sum = _C.moe_sum
 
-__all__ = ["moe_sum", "moe_plan_riders", "moe_balance_blocks", "moe_gemm_slot_rows", "topk_softmax", "moe_align_block_size", "topk_softmax_renorm",
+__all__ = ["moe_sum", "moe_plan_riders", "moe_plan_blocks", "moe_balance_blocks", "moe_gemm_slot_rows", "topk_softmax", "moe_align_block_size", "topk_softmax_renorm",
            "moe_align_block_size_filled", "moe_grouped_gemm", "fused_topk_align", "grouped_topk"]

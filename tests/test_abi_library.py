@@ -279,3 +279,25 @@ def test_rider_entry_points_validate_arguments_without_gpu(lib):
     assert gemm(layout=1) == UNSUPPORTED
     assert gemm(dt=0) == UNSUPPORTED
     assert gemm(valid=0) == OK
+
+
+def test_plan_blocks_validates_arguments_without_gpu(lib):
+    i64, ci, vp = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p
+    buf = ctypes.create_string_buffer(256)
+    p = ctypes.cast(buf, vp)
+    q = vp(p.value + 128)
+    null = vp(None)
+    INVALID, UNSUPPORTED, OK = -1, -2, 0
+
+    def plan(**kw):
+        return lib.sarathi_moe_plan_blocks(
+            kw.get("src", p), kw.get("dst", q), p, p, i64(kw.get("len", 512)), ci(kw.get("e", 8)),
+            ci(kw.get("bm", 256)), ci(4), kw.get("riders", p), i64(kw.get("riders_len", 2)), null)
+    assert plan(src=null) == INVALID
+    assert plan(dst=p) == INVALID               # in place
+    assert plan(riders=null) == INVALID
+    assert plan(riders_len=1) == INVALID        # one entry per slot block
+    assert plan(e=0) == INVALID
+    assert plan(bm=64) == UNSUPPORTED
+    assert plan(e=2000) == UNSUPPORTED
+    assert plan(len=0, riders_len=0) == OK

@@ -518,6 +518,79 @@ def test_riders_with_chosen_expert_loads(ops, dev, loads):
         assert torch.equal(with_r, base), (mul, silu)
 
 
+def _expected_plan(s, e, p, num_valid, bm=256):
+    """What sarathi_moe_plan_blocks documents: per expert, riders on the greedy layout, or the
+    even fill over the two halves of each block and no riders."""
+    s, e = s.tolist(), e.tolist()
+    live = min(int(p[0]), len(s)) // bm
+    out = list(s[:live * bm]) + [num_valid] * (len(s) - live * bm)
+    ride = [-1] * ((len(s) + bm - 1) // bm)
+    b = 0
+    while b < live:
+        last = b
+        while last + 1 < live and e[last + 1] == e[b]:
+            last += 1
+        nb = last - b + 1
+        slots = [x for x in s[b * bm:(last + 1) * bm] if x < num_valid]
+        valid_last = len(slots) - (nb - 1) * bm
+        tiles_last = (valid_last + 31) // 32
+        if nb > 1 and tiles_last <= nb - 1:
+            ride[last] = -2
+            for j in range(tiles_last):
+                ride[b + j] = last * bm + 32 * j
+        else:
+            tiles = (len(slots) + 31) // 32
+            ranges = 2 * nb
+            at = 0
+            for j in range(ranges):
+                mine = (tiles // ranges + (1 if j < tiles % ranges else 0)) * 32
+                take = slots[at:at + mine]
+                at += mine
+                out[b * bm + j * 128:b * bm + (j + 1) * 128] = take + [num_valid] * (128 - len(take))
+        b = last + 1
+    return out, ride
+
+
+@pytest.mark.parametrize("loads", [
+    (1024 + 33, 257, 0, 255, 512, 31),
+    (8 * 256 + 255, 0, 0, 1),
+    (8 * 256 + 256, 3 * 256 + 97, 2 * 256 + 65),
+    (256 + 32, 256 + 33, 512 + 64, 512 + 65),
+    (640, 650, 630, 600, 700, 640, 1, 300),
+])
+def test_moe_plan_blocks_matches_its_definition_and_keeps_the_bits(ops, dev, loads):
+    """moe_plan_blocks: riders for the experts whose last block fits onto their full blocks, the
+    even fill for the others, in one launch; the GEMM on its outputs has the bits of the GEMM on
+    moe_align_block_size's."""
+    bm, E, N, K = 256, len(loads), 520, 192
+    g = gen(sum(loads) + 1)
+    order = torch.cat([torch.full((n,), x, dtype=torch.int32) for x, n in enumerate(loads)])
+    ids = order[torch.randperm(order.numel(), generator=g)].view(-1, 1)
+    T = ids.numel()
+    n = T + E * (bm - 1)
+    s = torch.full((n,), T, dtype=torch.int32)
+    e = torch.zeros(((n + bm - 1) // bm,), dtype=torch.int32)
+    p = torch.zeros((1,), dtype=torch.int32)
+    c_oracle.moe_align_block_size(ids, E, bm, s, e, p)
+    sd, ed, pd = s.to(dev), e.to(dev), p.to(dev)
+    planned = torch.full_like(sd, -7)
+    riders = torch.full((e.numel(),), 99, dtype=torch.int32, device=dev)
+    ops.moe_ops.moe_plan_blocks(sd, planned, ed, pd, E, bm, T, riders)
+    want_sorted, want_ride = _expected_plan(s, e, p, T)
+    assert riders.cpu().tolist() == want_ride
+    assert planned.cpu().tolist() == want_sorted
+    A = randn((T, K), g, torch.bfloat16, std=0.5).to(dev)
+    Bw = randn((E, N, K), g, torch.bfloat16, std=0.5).to(dev)
+    wd = torch.rand((T, 1), generator=g).to(dev)
+    for mul, silu in ((True, False), (False, True)):
+        cols = N // 2 if silu else N
+        base = torch.full((T, 1, cols), 7.0, dtype=torch.bfloat16, device=dev)
+        got = torch.full((T, 1, cols), -3.0, dtype=torch.bfloat16, device=dev)
+        ops.moe_ops.moe_grouped_gemm(A, Bw, base, wd, sd, ed, pd, T, bm, 1, mul, False, N, silu)
+        ops.moe_ops.moe_grouped_gemm(A, Bw, got, wd, planned, ed, pd, T, bm, 1, mul, False, N, silu, riders)
+        assert torch.equal(got, base), (mul, silu)
+
+
 def test_fused_moe_same_bits_with_and_without_riders(ops, dev, monkeypatch):
     import importlib
     from sarathi_amd import layers
@@ -532,5 +605,7 @@ def test_fused_moe_same_bits_with_and_without_riders(ops, dev, monkeypatch):
     monkeypatch.setattr(fm, "RIDERS", False)
     base = layers.fused_moe(x, w1, w2, logits, k, True, override_config=cfg)
     monkeypatch.setattr(fm, "RIDERS", True)
-    got = layers.fused_moe(x, w1, w2, logits, k, True, override_config=cfg)
-    assert torch.equal(got, base)
+    for even_rest in (False, True):
+        monkeypatch.setattr(fm, "RIDERS_EVEN_REST", even_rest)
+        got = layers.fused_moe(x, w1, w2, logits, k, True, override_config=cfg)
+        assert torch.equal(got, base), even_rest
