@@ -8,7 +8,8 @@ rule could use, so that a rule added later is exercised on both sides without a 
 Each case goes through the op namespace -> C ABI and is compared with the oracle (rotary: bit for
 bit; norms: the dtype tolerance of the dense-op tests) or, for the fused append, bit for bit with
 the two stand-alone ops.  The activations, whose only rule is whole vectors or not, get a smaller
-sweep over widths, strides and dtypes.
+sweep over widths, strides and dtypes, and the grouped GEMM one over expert loads, for the per-expert
+choice between riders and the even fill of its slot blocks.
 """
 import os
 import random
@@ -218,3 +219,50 @@ def test_activation_sweep_matches_oracle(ops, dev, case):
     getattr(ops.activation_ops, name)(gotg, xg.to(dev))
     tol["max_mismatch_frac"] = max(tol["max_mismatch_frac"], 2e-2)
     assert_close_dtype(gotg, wantg, **tol)
+
+
+PLAN_CASES = 24 * _SCALE
+
+
+@pytest.mark.parametrize("case", range(PLAN_CASES))
+def test_planned_blocks_sweep_same_bits_as_plain_gemm(ops, dev, case):
+    """The grouped GEMM at 256-slot blocks with its blocks planned per expert (riders or the even
+    fill) against the same GEMM on moe_align_block_size's own layout, bit for bit: expert counts,
+    top-k, skewed and uniform expert loads, ragged N, all three epilogues, both 16-bit dtypes."""
+    rng = random.Random(8000 + case + _OFFSET)
+    E = rng.choice([2, 4, 8, 16, 24])
+    k = rng.choice([kk for kk in (1, 2, 4) if kk <= E])
+    per_expert = rng.choice([90, 200, 256, 257, 290, 400, 520, 545, 800, 1030, 1300])
+    T = max(1, per_expert * E // k + rng.randint(-7, 7))
+    N = 8 * rng.randint(32, 140)
+    K = 64 * rng.randint(1, 6)
+    dtype = rng.choice([torch.bfloat16, torch.float16])
+    mul, silu = rng.choice([(False, False), (True, False), (False, True)])
+    g = gen(9000 + case)
+    logits = torch.randn((T, E), generator=g, dtype=torch.float32)
+    if rng.random() < 0.5:                       # some experts hot, some nearly idle
+        logits += torch.randn((E,), generator=g) * rng.choice([0.3, 1.0])
+    weights, ids = torch.topk(torch.softmax(logits, dim=-1), k, dim=-1)
+    ids = ids.to(torch.int32).to(dev)
+    wd = weights.contiguous().to(dev)
+    bm = 256
+    n_sorted = T * k + E * (bm - 1)
+    sd = torch.empty((n_sorted,), dtype=torch.int32, device=dev)
+    ed = torch.zeros(((n_sorted + bm - 1) // bm,), dtype=torch.int32, device=dev)
+    pd = torch.empty((1,), dtype=torch.int32, device=dev)
+    ops.moe_ops.moe_align_block_size_filled(ids, E, bm, sd, ed, pd)
+    planned = torch.empty_like(sd)
+    riders = torch.empty((ed.numel(),), dtype=torch.int32, device=dev)
+    ops.moe_ops.moe_plan_blocks(sd, planned, ed, pd, E, bm, T * k, riders)
+    # every slot is still there exactly once
+    live = int(pd.item())
+    kept = planned[:live][planned[:live] < T * k]
+    assert torch.equal(torch.sort(kept).values, torch.arange(T * k, dtype=torch.int32, device=dev))
+    A = randn((T, K), g, dtype, std=0.5).to(dev)
+    Bw = randn((E, N, K), g, dtype, std=0.5).to(dev)
+    cols = N // 2 if silu else N
+    base = torch.full((T, k, cols), 7.0, dtype=dtype, device=dev)
+    got = torch.full((T, k, cols), -3.0, dtype=dtype, device=dev)
+    ops.moe_ops.moe_grouped_gemm(A, Bw, base, wd, sd, ed, pd, T * k, bm, k, mul, False, N, silu)
+    ops.moe_ops.moe_grouped_gemm(A, Bw, got, wd, planned, ed, pd, T * k, bm, k, mul, False, N, silu, riders)
+    assert torch.equal(got, base)
