@@ -414,7 +414,8 @@ int sarathi_moe_grouped_gemm_riders(const void* a, const void* b, void* c, const
  * `sorted_in`, not the same memory) and `riders` (one int32 per slot block, at least
  * ceil(sorted_len / block_m)) then go to sarathi_moe_grouped_gemm_riders together with the
  * unchanged expert_ids and num_tokens_post_padded.  `pad_value` is the padding id
- * (num_valid_tokens).  Same GEMM results bit for bit.
+ * (num_valid_tokens); `sorted_in` must carry it in every unused slot of the live blocks
+ * (sarathi_moe_align_block_size with fill_pad = 1).  Same GEMM results bit for bit.
  */
 int sarathi_moe_plan_blocks(const int32_t* sorted_in, int32_t* sorted_out, const int32_t* expert_ids,
                             const int32_t* num_tokens_post_padded, int64_t sorted_len,

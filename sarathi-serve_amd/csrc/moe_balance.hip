@@ -130,8 +130,9 @@ __global__ __launch_bounds__(256) void moe_plan_blocks_kernel(
   if (b1 < 0) return;  // the expert has no block (uniform)
   const int nb = b1 - b0 + 1;
   const int64_t base = (int64_t)b0 * block;
-  int c = 0;
-  for (int i = tid; i < block; i += 256) c += sorted_in[(int64_t)b1 * block + i] != pad_value;
+  int c = 0;  // ids are 0 .. pad_value - 1, padding is pad_value
+  for (int i = tid; i < block; i += 256)
+    c += (uint32_t)sorted_in[(int64_t)b1 * block + i] < (uint32_t)pad_value;
   if (c) atomicAdd(&valid_last, c);
   __syncthreads();
   const int tiles_last = (valid_last + granule - 1) / granule;
