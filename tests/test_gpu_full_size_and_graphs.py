@@ -256,7 +256,8 @@ def test_mixtral_expert_gemms_full_size(ops, dev):
     bit for bit; (2) doubling the activations doubles every output exactly (power-of-two scaling
     commutes with every rounding as long as nothing overflows); (3) a random sample of outputs
     against float64 dot products of the gathered rows; (4) the gated epilogue against the separate
-    activation kernel."""
+    activation kernel; (5) the kernel with riders on slot blocks planned per expert against (1)
+    and (4), bit for bit."""
     from sarathi_amd import layers
     T, E, k, H, I = 4096, 8, 2, 4096, 14336
     bf = torch.bfloat16
@@ -293,6 +294,17 @@ def test_mixtral_expert_gemms_full_size(ops, dev):
     ops.activation_ops.silu_and_mul(act, plain)
     assert torch.equal(run(x, w1, False, True), act)
     assert torch.equal(run(x, packed_w1, True, True), act)
+    # (5) slot blocks planned per expert (riders, even fill): same bits, both epilogues
+    if bm == 256:
+        planned = torch.empty_like(s)
+        riders = torch.empty((e.numel(),), dtype=torch.int32, device=dev)
+        ops.moe_ops.moe_plan_blocks(s, planned, e, p, E, bm, T * k, riders)
+        assert bool((riders >= 0).any()), "this routing has tiles that ride"
+        for gated, want_c in ((False, plain), (True, act)):
+            c = torch.full_like(want_c, 3.0)
+            ops.moe_ops.moe_grouped_gemm(x, w1, c, tw, planned, e, p, T * k, bm, k, False, False, 2 * I,
+                                         gated, riders)
+            assert torch.equal(c, want_c), gated
 
 
 def test_fused_moe_with_riders_under_hip_graph_capture(ops, dev, monkeypatch):
