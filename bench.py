@@ -637,7 +637,7 @@ def main():
             w1.fill_(0.0078125)
             w2.fill_(0.0078125)
         forward = {}
-        for Tn in (16, 1024, 2048, 4096):
+        for Tn in (16, 1024, 2048, 2304, 4096):
             x = torch.randn((Tn, Hm), device=dev, dtype=torch.float32).to(bf16)
             if args.moe_data == "constant":
                 x.fill_(0.0078125)
