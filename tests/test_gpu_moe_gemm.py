@@ -609,3 +609,22 @@ def test_fused_moe_same_bits_with_and_without_riders(ops, dev, monkeypatch):
         monkeypatch.setattr(fm, "RIDERS_EVEN_REST", even_rest)
         got = layers.fused_moe(x, w1, w2, logits, k, True, override_config=cfg)
         assert torch.equal(got, base), even_rest
+
+
+def test_fused_moe_commutes_with_a_permutation_of_the_tokens(ops, dev):
+    """A token's output does not depend on where its slots land in the sorted layout (which block,
+    which tile, riding or not): permuting the batch permutes the output, bit for bit, through
+    routing, slot sort, block planning, both GEMMs and the top-k sum."""
+    from sarathi_amd import layers
+    T, E, k, H, I = 1500, 8, 2, 512, 768
+    g = gen(77)
+    x = randn((T, H), g, torch.bfloat16, std=0.5).to(dev)
+    w1 = randn((E, 2 * I, H), g, torch.bfloat16, std=0.05).to(dev)
+    w2 = randn((E, H, I), g, torch.bfloat16, std=0.05).to(dev)
+    logits = torch.randn((T, E), generator=g, dtype=torch.float32).to(dev)
+    perm = torch.randperm(T, generator=g).to(dev)
+    for cfg in ({"BLOCK_SIZE_M": 256}, {"BLOCK_SIZE_M": 64}):
+        out = layers.fused_moe(x, w1, w2, logits, k, True, override_config=cfg)
+        out_p = layers.fused_moe(x[perm].contiguous(), w1, w2, logits[perm].contiguous(), k, True,
+                                 override_config=cfg)
+        assert torch.equal(out_p, out[perm]), cfg
